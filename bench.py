@@ -1,0 +1,335 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused per-layer kernels on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only NAME] [--no-cpu] [--warm]
+
+Prints ONE JSON line.  The headline workload is the fused add-bias + residual + RMSNorm in fp16 at
+2048 tokens x 4096 hidden (one step = one launch over one batch); `kernels` carries the same
+measurement for every kernel of the path at its LLaMA-2-7B shape.
+
+Method
+  * inputs are synthetic (torch RNG on the device), resident in HBM before the timed region;
+  * every launch works on the next of R buffer sets, R chosen so the sets together exceed 1 GiB:
+    successive launches cannot be served from the 256 MB last-level cache ("cold"; --warm disables
+    the rotation and is reported separately, never as `value`);
+  * K launches are issued back to back on a private stream between two HIP events recorded on that
+    stream, bracketed by synchronize on both sides; ms_per_step is the host wall clock over the
+    same region, roofline.achieved uses the event time / K (so it includes the gaps between
+    consecutive launches and is a lower bound on the in-kernel rate);
+  * achieved = algorithmic bytes per launch (each operand once: compulsory reads + writes) / time.
+  * cpu_baseline: the C oracle (a port of the reference's CPU test functions) timed on the host
+    cores of the same machine, on the same workload shape, single thread plus an OpenMP run.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published peak
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--only", default=None, help="run a single workload by name")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--warm", action="store_true", help="also report cache-warm (no rotation) rates")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline leg")
+    return ap.parse_args()
+
+
+# --------------------------------------------------------------------------- workloads
+
+class Workload:
+    """One kernel at one shape: R rotating buffer sets and a launch(i) closure."""
+    name = ""
+    dtype = ""
+    tokens = 0
+    bytes_per_launch = 0
+    kernel_symbol = ""
+
+    def sets_for(self, set_bytes, rotate):
+        if not rotate:
+            return 1
+        return max(2, int((1 << 30) // max(set_bytes, 1)) + 1)
+
+
+def make_workloads(torch, ops, rotate):
+    dev = "cuda"
+    W = []
+
+    def norm(name, tokens, hidden, tdtype, fused):
+        w = Workload()
+        es = 2 if tdtype == torch.float16 else 4
+        w.name, w.dtype, w.tokens = name, ("f16" if es == 2 else "f32"), tokens
+        w.kernel_symbol = "fused_norm_rows"
+        if fused:
+            w.bytes_per_launch = 4 * tokens * hidden * es + 2 * hidden * es
+            set_bytes = 2 * tokens * hidden * es
+        else:
+            w.bytes_per_launch = 2 * tokens * hidden * es + hidden * es
+            set_bytes = tokens * hidden * es
+        R = w.sets_for(set_bytes, rotate)
+        outs = [torch.randn((tokens, hidden), device=dev, dtype=torch.float32).to(tdtype) for _ in range(R)]
+        ress = [torch.randn((tokens, hidden), device=dev, dtype=torch.float32).to(tdtype) for _ in range(R)] if fused else None
+        bias = (0.02 * torch.randn(hidden, device=dev)).to(tdtype) if fused else None
+        gamma = (0.5 + torch.rand(hidden, device=dev)).to(tdtype)
+        w.sets = R
+
+        def launch(i):
+            j = i % R
+            if fused:
+                ops.fused_add_bias_residual_rmsnorm(ress[j], outs[j], bias, gamma, 1e-5)
+            else:
+                ops.rmsnorm(outs[j], gamma, 1e-5)
+
+        def reset():
+            # the kernel works in place: refresh the values so repeated launches stay finite
+            for t in outs:
+                t.normal_()
+            if fused:
+                for t in ress:
+                    t.normal_()
+
+        w.launch, w.reset = launch, reset
+        w.config = {"tokens": tokens, "hidden": hidden}
+        return w
+
+    def embedding():
+        w = Workload()
+        tokens, hidden, vocab = 8192, 4096, 32000
+        w.name, w.dtype, w.tokens = "embedding_f16_8192x4096_v32000", "f16", tokens
+        w.kernel_symbol = "gather_rows_vec"
+        w.bytes_per_launch = 2 * tokens * hidden * 2 + tokens * 4
+        table = (0.02 * torch.randn((vocab, hidden), device=dev)).to(torch.float16)
+        R = w.sets_for(tokens * hidden * 2, rotate)
+        ids = [torch.randint(0, vocab, (tokens,), device=dev, dtype=torch.int32) for _ in range(R)]
+        outs = [torch.empty((tokens, hidden), device=dev, dtype=torch.float16) for _ in range(R)]
+        w.sets = R
+        w.launch = lambda i: ops.input_embedding(ids[i % R], outs[i % R], table)
+        w.reset = lambda: None
+        w.config = {"tokens": tokens, "hidden": hidden, "vocab": vocab}
+        return w
+
+    def qkv():
+        w = Workload()
+        batch, seq, hn, kvn, hs = 8, 512, 32, 32, 128
+        g = torch.Generator(device="cpu").manual_seed(0)
+        lens = torch.randint(256, 513, (batch,), generator=g, dtype=torch.int32)
+        tokens = int(lens.sum())
+        w.name, w.dtype, w.tokens = "qkv_bias_rope_transpose_f16_b8_s512", "f16", tokens
+        w.kernel_symbol = "qkv_rope_vec"
+        w.bytes_per_launch = tokens * (2 * (hn + 2 * kvn) * hs * 2 + 4) + (hn + 2 * kvn) * hs * 2 + 2 * batch * 4
+        lens_d = lens.to(dev)
+        po = torch.zeros((batch, seq), device=dev, dtype=torch.int32)
+        cum = torch.zeros((batch + 1,), device=dev, dtype=torch.int32)
+        ops.cal_padding_offset(po, cum, lens_d)
+        hist = torch.zeros(batch, device=dev, dtype=torch.int32)
+        bias = (0.02 * torch.randn((hn + 2 * kvn) * hs, device=dev)).to(torch.float16)
+        set_bytes = tokens * (hn + 2 * kvn) * hs * 2 + 3 * batch * hn * seq * hs * 2
+        R = w.sets_for(set_bytes, rotate)
+        ins = [torch.randn((tokens, hn + 2 * kvn, hs), device=dev).to(torch.float16) for _ in range(R)]
+        outs = [[torch.zeros((batch, n, seq, hs), device=dev, dtype=torch.float16) for n in (hn, kvn, kvn)]
+                for _ in range(R)]
+        w.sets = R
+
+        def launch(i):
+            j = i % R
+            ops.add_fused_qkv_bias_transpose_and_rope(outs[j][0], outs[j][1], outs[j][2], ins[j], bias, po, hist,
+                                                      lens_d, 128, 10000.0)
+
+        w.launch, w.reset = launch, (lambda: None)
+        w.config = {"batch": batch, "max_seq": seq, "valid_tokens": tokens, "heads": "32q/32kv", "head_dim": hs}
+        return w
+
+    def swiglu(tokens, tag):
+        w = Workload()
+        inter = 11008
+        w.name, w.dtype, w.tokens = "swiglu_f16_%s_%dx%d" % (tag, tokens, inter), "f16", tokens
+        w.kernel_symbol = "swiglu_vec"
+        w.bytes_per_launch = tokens * 3 * inter * 2
+        R = w.sets_for(w.bytes_per_launch, rotate)
+        ins = [torch.randn((tokens, 2, inter), device=dev).to(torch.float16) for _ in range(R)]
+        outs = [torch.empty((tokens, inter), device=dev, dtype=torch.float16) for _ in range(R)]
+        w.sets = R
+        w.launch = lambda i: ops.act(ins[i % R], outs[i % R])
+        w.reset = lambda: None
+        w.config = {"tokens": tokens, "inter": inter}
+        return w
+
+    makers = [
+        ("fused_add_bias_residual_rmsnorm_f16_2048x4096",
+         lambda: norm("fused_add_bias_residual_rmsnorm_f16_2048x4096", 2048, 4096, torch.float16, True)),
+        ("rmsnorm_f32_64x4096", lambda: norm("rmsnorm_f32_64x4096", 64, 4096, torch.float32, False)),
+        ("rmsnorm_f32_16384x4096", lambda: norm("rmsnorm_f32_16384x4096", 16384, 4096, torch.float32, False)),
+        ("embedding_f16_8192x4096_v32000", embedding),
+        ("qkv_bias_rope_transpose_f16_b8_s512", qkv),
+        ("swiglu_f16_prefill_8192x11008", lambda: swiglu(8192, "prefill")),
+        ("swiglu_f16_decode_256x11008", lambda: swiglu(256, "decode")),
+    ]
+    return makers
+
+
+# --------------------------------------------------------------------------- timing
+
+def time_workload(torch, w, steps, warmup, stream):
+    with torch.cuda.stream(stream):
+        w.reset()
+        for i in range(warmup):
+            w.launch(i)
+        stream.synchronize()
+        w.reset()
+        torch.cuda.synchronize()
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        t0 = time.perf_counter()
+        e0.record(stream)
+        for i in range(steps):
+            w.launch(i)
+        e1.record(stream)
+        stream.synchronize()
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+    wall_ms = (t1 - t0) * 1e3 / steps
+    event_ms = e0.elapsed_time(e1) / steps
+    return wall_ms, event_ms
+
+
+def per_launch_event_ms(torch, w, steps, stream):
+    """Average of per-launch (event, launch, event) brackets: excludes most of the gap between
+    consecutive launches; reported next to the region average."""
+    n = min(steps, 100)
+    with torch.cuda.stream(stream):
+        w.reset()
+        torch.cuda.synchronize()
+        evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n)]
+        for i, (a, b) in enumerate(evs):
+            a.record(stream)
+            w.launch(i)
+            b.record(stream)
+        stream.synchronize()
+    ts = sorted(a.elapsed_time(b) for a, b in evs)
+    return sum(ts) / len(ts), ts[len(ts) // 2]
+
+
+def measure(torch, w, steps, warmup, stream):
+    wall_ms, event_ms = time_workload(torch, w, steps, warmup, stream)
+    pl_mean, pl_median = per_launch_event_ms(torch, w, steps, stream)
+    gbs = w.bytes_per_launch / (event_ms * 1e-3) / 1e9
+    return {
+        "workload": w.name, "dtype": w.dtype, "tokens": w.tokens, "buffer_sets": w.sets,
+        "algorithmic_bytes": w.bytes_per_launch,
+        "ms_per_step_wall": wall_ms, "ms_per_launch_events": event_ms,
+        "ms_per_launch_bracketed_mean": pl_mean, "ms_per_launch_bracketed_median": pl_median,
+        "GBps": gbs, "frac_of_hbm_peak": gbs / HBM_PEAK_GBS,
+        "GBps_bracketed_median": w.bytes_per_launch / (pl_median * 1e-3) / 1e9,
+        "tokens_per_s": w.tokens / (event_ms * 1e-3),
+    }
+
+
+# --------------------------------------------------------------------------- CPU baseline
+
+def cpu_baseline(budget_s):
+    """Times the C oracle (port of the reference's CPU functions) on the headline workload shape."""
+    import numpy as np
+    sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+    from oracle import load
+    o = load()
+    tokens, hidden = 2048, 4096
+    r = np.random.default_rng(0)
+    out = r.standard_normal((tokens, hidden)).astype(np.float16)
+    res = r.standard_normal((tokens, hidden)).astype(np.float16)
+    bias = (0.02 * r.standard_normal(hidden)).astype(np.float16)
+    gamma = r.uniform(0.5, 1.5, hidden).astype(np.float16)
+    nbytes = 4 * tokens * hidden * 2 + 2 * hidden * 2
+
+    def run(threads, budget):
+        o.set_threads(threads)
+        lib = o.lib
+        times = []
+        t_end = time.perf_counter() + budget
+        a, b = out.copy(), res.copy()
+        while len(times) < 3 or (time.perf_counter() < t_end and len(times) < 50):
+            a[...] = out
+            b[...] = res
+            t0 = time.perf_counter()
+            lib.isp_oracle_fused_norm_f16(b.ctypes.data, a.ctypes.data, bias.ctypes.data, gamma.ctypes.data,
+                                          1e-5, tokens, hidden, 0)
+            times.append(time.perf_counter() - t0)
+        o.set_threads(1)
+        times.sort()
+        return times[len(times) // 2], len(times)
+
+    t1, n1 = run(1, budget_s * 0.6)
+    cores = min(16, o.max_threads())
+    tn, nn = run(cores, budget_s * 0.4)
+    return {
+        "value": nbytes / t1 / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+        "sample": "full workload (2048x4096 fp16 fused add-bias+residual+RMSNorm), median of %d runs" % n1,
+        "tokens_per_s": tokens / t1,
+        "openmp": {"value": nbytes / tn / 1e9, "unit": "GB/s", "cores": cores, "tokens_per_s": tokens / tn,
+                   "runs": nn},
+    }
+
+
+# --------------------------------------------------------------------------- main
+
+def main():
+    a = parse()
+    if a.gpus != 1:
+        print("bench.py: this build measures one GPU only; --gpus %d is not supported (use --gpus 1)" % a.gpus,
+              file=sys.stderr)
+        sys.exit(2)
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU available; the kernels have no CPU path", file=sys.stderr)
+        sys.exit(3)
+    from inferspore_amd import capi, ops
+    capi.check(capi.lib().isp_init(), "isp_init")
+    torch.manual_seed(0)
+    stream = torch.cuda.Stream()
+
+    results, warm = [], {}
+    for name, make in make_workloads(torch, ops, True):
+        if a.only and a.only != name:
+            continue
+        w = make()
+        results.append(measure(torch, w, a.steps, a.warmup, stream))
+        del w
+        torch.cuda.empty_cache()
+    if a.warm:
+        for name, make in make_workloads(torch, ops, False):
+            if a.only and a.only != name:
+                continue
+            w = make()
+            m = measure(torch, w, a.steps, a.warmup, stream)
+            warm[name] = {"GBps": m["GBps"], "ms_per_launch_events": m["ms_per_launch_events"]}
+            del w
+            torch.cuda.empty_cache()
+    head = results[0]
+    line = {
+        "metric": "HBM GB/s & % of peak per fused kernel at LLaMA-2-7B shapes; tokens/sec",
+        "value": head["GBps"], "unit": "GB/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": head["ms_per_step_wall"], "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f16 storage / f32 arithmetic", "data": "synthetic",
+        "config": {"workload": head["workload"], "tokens_per_s": head["tokens_per_s"],
+                   "cache": "cold (rotating %d buffer sets > 1 GiB)" % head["buffer_sets"]},
+        "roofline": {"bound": "hbm", "achieved": head["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": head["GBps"] / HBM_PEAK_GBS, "traffic": None,
+                     "kernel": "fused_norm_rows<__half, 2, 4>",
+                     "algorithmic_bytes_per_launch": head["algorithmic_bytes"],
+                     "avg_launch_ms": head["ms_per_launch_events"]},
+        "kernels": results,
+    }
+    if warm:
+        line["warm_cache"] = warm
+    if not a.no_cpu:
+        line["cpu_baseline"] = cpu_baseline(a.cpu_seconds)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,146 @@
+/*
+ * inferspore_amd.h -- C ABI of the MI355X (gfx950) implementation of InferSpore's fused
+ * per-layer kernels.
+ *
+ * This is the drop-in boundary: every entry point takes raw device pointers, plain integers and a
+ * HIP stream, launches hand-written HIP kernels asynchronously on that stream, allocates nothing,
+ * keeps no state and returns 0 or a negative isp_status.  The C++ `launch*` templates declared
+ * under include/src/kernels/ (same names and parameter lists as the reference's) are thin shims
+ * over these functions; a binding from any other language needs only this header.
+ *
+ * Each declaration names the reference interface it replaces (paths relative to the
+ * m0dulo/InferSpore checkout).
+ *
+ * Conventions
+ *   - all tensors are dense, row-major, device-resident; `_f16` = IEEE binary16 storage with fp32
+ *     arithmetic and a single rounding per stored value, `_f32` = binary32 throughout;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream, which is what the
+ *     reference's launchers use);
+ *   - pointers documented "may be NULL" are optional operands; any other NULL pointer gives
+ *     ISP_ERR_NULL_POINTER (unless the call has no work to do: zero tokens returns ISP_OK first);
+ *   - 16-byte aligned pointers and vector-friendly extents take the fast 128-bit path; anything
+ *     else is routed to a slower scalar kernel with identical results.
+ */
+#ifndef INFERSPORE_AMD_H
+#define INFERSPORE_AMD_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum isp_status {
+    ISP_OK = 0,
+    ISP_ERR_NULL_POINTER = -1, /* a required pointer is NULL */
+    ISP_ERR_BAD_SHAPE = -2,    /* negative / inconsistent extents */
+    ISP_ERR_UNSUPPORTED = -3,  /* extents outside what the kernels implement */
+    ISP_ERR_LAUNCH = -4,       /* HIP reported an error at launch; see isp_last_hip_error() */
+    ISP_ERR_DEVICE = -5        /* no usable gfx950 device */
+} isp_status;
+
+/* flag bits for isp_fused_add_bias_residual_rmsnorm_* */
+#define ISP_NORM_RESIDUAL_EXCLUDES_BIAS 1u
+
+typedef void* isp_stream_t; /* hipStream_t */
+
+/* Library identification and diagnostics (no reference counterpart). */
+const char* isp_version(void);
+const char* isp_strerror(int status);
+/* hipError_t of the most recent failed launch on the calling thread (0 if none). */
+int isp_last_hip_error(void);
+/* Checks that the current HIP device exists and is a gfx950; optional, the kernels need no set-up. */
+int isp_init(void);
+
+/*
+ * Input-embedding gather: out[t, :] = table[ids[t], :].
+ * Replaces launchInputEmbedding<T> (src/kernels/input_embedding.h:6-9, .cu:25-45).
+ *   ids [tokens] int32, table [vocab, hidden], out [tokens, hidden].
+ * `vocab` > 0 enables a bounds check (rows whose id is outside [0, vocab) are written as zeros
+ * instead of reading out of bounds); vocab == 0 reproduces the reference's unchecked gather.
+ */
+int isp_embedding_f16(const int32_t* ids, void* out, const void* table, int tokens, int hidden,
+                      int vocab, isp_stream_t stream);
+int isp_embedding_f32(const int32_t* ids, void* out, const void* table, int tokens, int hidden,
+                      int vocab, isp_stream_t stream);
+
+/*
+ * Padding-offset builder.
+ * Replaces launchCalPaddingoffset (src/kernels/cal_paddingoffset.h:8-11, .cu:18-60).
+ *   input_lengths [batch]; padding_offset [batch, max_q_len] (only the first sum(lengths) entries
+ *   are written); cum_seqlens [batch + 1].
+ */
+int isp_cal_padding_offset(int32_t* padding_offset, int32_t* cum_seqlens,
+                           const int32_t* input_lengths, int batch, int max_q_len,
+                           isp_stream_t stream);
+
+/*
+ * RMSNorm, in place: x := x * rsqrt(mean(x^2) + eps) * gamma.
+ * The reference reaches this through launchFusedAddBiasResidualRMSNorm<T> with a NULL residual and
+ * bias (src/kernels/fused_addresidual_norm.cu:51,56,68); same kernel here.
+ *   x [tokens, hidden], gamma [hidden].
+ */
+int isp_rmsnorm_f32(void* x, const void* gamma, float eps, int tokens, int hidden,
+                    isp_stream_t stream);
+int isp_rmsnorm_f16(void* x, const void* gamma, float eps, int tokens, int hidden,
+                    isp_stream_t stream);
+
+/*
+ * Fused add-bias + residual + RMSNorm, in place on both tensors.
+ * Replaces launchFusedAddBiasResidualRMSNorm<T> (src/kernels/fused_addresidual_norm.h:9-15,
+ * .cu:32-98,143-170).
+ *   x            = decoder_out + residual + bias
+ *   residual    := x                       (flags == 0)
+ *   residual    := decoder_out + residual  (ISP_NORM_RESIDUAL_EXCLUDES_BIAS: the reference's
+ *                                           literal store order, .cu:62-67)
+ *   decoder_out := gamma * x * rsqrt(mean(x^2) + eps)
+ *   residual, decoder_out [tokens, hidden]; bias, gamma [hidden]; residual and bias may be NULL.
+ */
+int isp_fused_add_bias_residual_rmsnorm_f32(void* residual, void* decoder_out, const void* bias,
+                                            const void* gamma, float eps, int tokens, int hidden,
+                                            unsigned flags, isp_stream_t stream);
+int isp_fused_add_bias_residual_rmsnorm_f16(void* residual, void* decoder_out, const void* bias,
+                                            const void* gamma, float eps, int tokens, int hidden,
+                                            unsigned flags, isp_stream_t stream);
+
+/*
+ * Fused QKV bias + rotate-half RoPE + head transpose + re-padding (prefill).
+ * Replaces launchAddFusedQKVBiasTransposeAndRoPE<T> (src/kernels/qkv_bias_and_RoPE.h:10-20,
+ * .cu:109-192,286-330).
+ *   qkv [token_num, head_num + 2 kv_head_num, head_size] packed (no padding);
+ *   bias [(head_num + 2 kv_head_num) * head_size], may be NULL;
+ *   padding_offset [token_num]; history_length, input_length [batch];
+ *   q [batch, head_num, seq_len, head_size]; k, v [batch, kv_head_num, seq_len, head_size].
+ * Token t lands at flat padded position p = t + padding_offset[t] (b = p / seq_len,
+ * s = p % seq_len) and is rotated at timestep history_length[b] + s.  Padded positions are not
+ * written.  A token whose p falls outside [0, batch * seq_len) is skipped (the reference would
+ * write out of bounds).  `max_position_embeddings` and `use_dynamic_ntk` are accepted and ignored,
+ * as in the reference (.cu:126-127).
+ */
+int isp_qkv_bias_rope_transpose_f32(void* q, void* k, void* v, const void* qkv, const void* bias,
+                                    const int32_t* padding_offset, const int32_t* history_length,
+                                    const int32_t* input_length, int batch, int seq_len,
+                                    int token_num, int head_num, int kv_head_num, int head_size,
+                                    int rotary_embedding_dim, float rotary_embedding_base,
+                                    int max_position_embeddings, int use_dynamic_ntk,
+                                    isp_stream_t stream);
+int isp_qkv_bias_rope_transpose_f16(void* q, void* k, void* v, const void* qkv, const void* bias,
+                                    const int32_t* padding_offset, const int32_t* history_length,
+                                    const int32_t* input_length, int batch, int seq_len,
+                                    int token_num, int head_num, int kv_head_num, int head_size,
+                                    int rotary_embedding_dim, float rotary_embedding_base,
+                                    int max_position_embeddings, int use_dynamic_ntk,
+                                    isp_stream_t stream);
+
+/*
+ * SwiGLU activation: out[t, i] = silu(in[t, 0, i]) * in[t, 1, i], silu(x) = x / (1 + exp(-x)).
+ * Replaces launchAct<T> (src/kernels/act_kernel.h:8-9, .cu:18-71).
+ *   in [tokens, 2, inter], out [tokens, inter].
+ */
+int isp_swiglu_f32(const void* in, void* out, int tokens, int inter, isp_stream_t stream);
+int isp_swiglu_f16(const void* in, void* out, int tokens, int inter, isp_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* INFERSPORE_AMD_H */

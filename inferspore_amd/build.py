@@ -1,0 +1,108 @@
+"""In-tree build of the gfx950 libraries with hipcc (no cmake, no JIT cache).
+
+    python -m inferspore_amd.build          # build everything
+    python -m inferspore_amd.build --clean
+
+Outputs (git-ignored, but they travel with the source tree to a GPU machine):
+    inferspore_amd/lib/libinferspore_amd.so     HIP kernels + the C ABI (include/inferspore_amd.h)
+    inferspore_amd/lib/libinferspore_launch.so  the C++ `launch*` shims over the C ABI
+    build/bin/test_*                            reference-style C++ call-site programs
+"""
+import argparse
+import concurrent.futures as cf
+import os
+import shutil
+import subprocess
+import sys
+
+PKG = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(PKG)
+CSRC = os.path.join(PKG, "csrc")
+LIBDIR = os.path.join(PKG, "lib")
+OBJDIR = os.path.join(ROOT, "build", "obj")
+BINDIR = os.path.join(ROOT, "build", "bin")
+INCLUDE = os.path.join(ROOT, "include")
+CPPTESTS = os.path.join(ROOT, "tests", "cpp")
+
+ARCH = "gfx950"
+# -packed-fp32-ops: keep the compiler from forming packed fp32 VALU instructions.
+HIPCC_FLAGS = [
+    "--offload-arch=" + ARCH, "-O3", "-std=c++17", "-fPIC", "-I" + INCLUDE, "-I" + CSRC,
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wall", "-Wno-unused-function",
+]
+
+LIB_KERNELS = os.path.join(LIBDIR, "libinferspore_amd.so")
+LIB_LAUNCH = os.path.join(LIBDIR, "libinferspore_launch.so")
+
+
+def _run(cmd):
+    p = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    out = "\n".join(l for l in p.stdout.splitlines()
+                    if "is not a recognized feature for this target" not in l)
+    if p.returncode != 0:
+        raise RuntimeError("command failed (%d): %s\n%s" % (p.returncode, " ".join(cmd), out))
+    return out
+
+
+def hipcc():
+    exe = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(exe):
+        raise RuntimeError("hipcc not found; the HIP libraries cannot be built")
+    return exe
+
+
+def _compile(src):
+    obj = os.path.join(OBJDIR, os.path.splitext(os.path.basename(src))[0] + ".o")
+    out = _run([hipcc()] + HIPCC_FLAGS + ["-c", src, "-o", obj])
+    return obj, out
+
+
+def build(verbose=False, jobs=8, cpp_tests=True):
+    for d in (LIBDIR, OBJDIR, BINDIR):
+        os.makedirs(d, exist_ok=True)
+    kernel_srcs = sorted(os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".hip"))
+    with cf.ThreadPoolExecutor(max_workers=jobs) as ex:
+        results = list(ex.map(_compile, kernel_srcs))
+    for obj, out in results:
+        if verbose and out.strip():
+            print(out)
+    objs = [o for o, _ in results]
+    _run([hipcc(), "--offload-arch=" + ARCH, "-shared", "-fPIC", "-o", LIB_KERNELS] + objs)
+
+    launch_src = os.path.join(CSRC, "launchers.cc")
+    if os.path.exists(launch_src):
+        _run([hipcc()] + HIPCC_FLAGS + ["-x", "hip", "-shared", launch_src, "-o", LIB_LAUNCH,
+                                        "-L" + LIBDIR, "-linferspore_amd", "-Wl,-rpath,$ORIGIN"])
+        if cpp_tests and os.path.isdir(CPPTESTS):
+            oracle_dir = os.path.join(ROOT, "oracle")
+            srcs = sorted(f for f in os.listdir(CPPTESTS) if f.endswith(".cc"))
+
+            def one(f):
+                exe = os.path.join(BINDIR, os.path.splitext(f)[0])
+                return _run([hipcc()] + HIPCC_FLAGS + [
+                    "-x", "hip", os.path.join(CPPTESTS, f), "-o", exe, "-I" + oracle_dir,
+                    "-L" + LIBDIR, "-linferspore_launch", "-linferspore_amd",
+                    "-L" + oracle_dir, "-lisp_oracle",
+                    "-Wl,-rpath," + LIBDIR, "-Wl,-rpath," + oracle_dir])
+
+            with cf.ThreadPoolExecutor(max_workers=jobs) as ex:
+                list(ex.map(one, srcs))
+    return LIB_KERNELS
+
+
+def clean():
+    for p in (LIB_KERNELS, LIB_LAUNCH):
+        if os.path.exists(p):
+            os.remove(p)
+    shutil.rmtree(os.path.join(ROOT, "build"), ignore_errors=True)
+
+
+if __name__ == "__main__":
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--clean", action="store_true")
+    ap.add_argument("-v", "--verbose", action="store_true")
+    a = ap.parse_args()
+    if a.clean:
+        clean()
+        sys.exit(0)
+    print(build(verbose=a.verbose))

@@ -1,0 +1,69 @@
+"""ctypes view of include/inferspore_amd.h.  Loading fails loudly when the library is not built."""
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libinferspore_amd.so")
+
+OK = 0
+ERR_NULL_POINTER = -1
+ERR_BAD_SHAPE = -2
+ERR_UNSUPPORTED = -3
+ERR_LAUNCH = -4
+ERR_DEVICE = -5
+NORM_RESIDUAL_EXCLUDES_BIAS = 1
+
+_vp, _i, _f, _u = C.c_void_p, C.c_int, C.c_float, C.c_uint
+
+# name -> (restype, argtypes); one entry per function declared in the public header
+SIGNATURES = {
+    "isp_version": (C.c_char_p, []),
+    "isp_strerror": (C.c_char_p, [_i]),
+    "isp_last_hip_error": (_i, []),
+    "isp_init": (_i, []),
+    "isp_embedding_f16": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp]),
+    "isp_embedding_f32": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp]),
+    "isp_cal_padding_offset": (_i, [_vp, _vp, _vp, _i, _i, _vp]),
+    "isp_rmsnorm_f32": (_i, [_vp, _vp, _f, _i, _i, _vp]),
+    "isp_rmsnorm_f16": (_i, [_vp, _vp, _f, _i, _i, _vp]),
+    "isp_fused_add_bias_residual_rmsnorm_f32": (_i, [_vp, _vp, _vp, _vp, _f, _i, _i, _u, _vp]),
+    "isp_fused_add_bias_residual_rmsnorm_f16": (_i, [_vp, _vp, _vp, _vp, _f, _i, _i, _u, _vp]),
+    "isp_qkv_bias_rope_transpose_f32": (_i, [_vp] * 8 + [_i] * 7 + [_f, _i, _i, _vp]),
+    "isp_qkv_bias_rope_transpose_f16": (_i, [_vp] * 8 + [_i] * 7 + [_f, _i, _i, _vp]),
+    "isp_swiglu_f32": (_i, [_vp, _vp, _i, _i, _vp]),
+    "isp_swiglu_f16": (_i, [_vp, _vp, _i, _i, _vp]),
+    "isp_tuning_norm_waves_per_row": (_i, [_i]),
+}
+
+_lib = None
+
+
+class IspError(RuntimeError):
+    def __init__(self, status, where):
+        self.status = status
+        msg = lib().isp_strerror(status).decode()
+        if status == ERR_LAUNCH:
+            msg += " (hipError %d)" % lib().isp_last_hip_error()
+        super().__init__("[inferspore_amd] %s failed: %s (status %d)" % (where, msg, status))
+
+
+def lib():
+    """The loaded C-ABI library.  Raises if it has not been built (python -m inferspore_amd.build)."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                "inferspore_amd: %s is missing -- build it with `python -m inferspore_amd.build`; "
+                "there is no fallback implementation" % LIB_PATH)
+        l = C.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(l, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = l
+    return _lib
+
+
+def check(status, where):
+    if status != OK:
+        raise IspError(status, where)

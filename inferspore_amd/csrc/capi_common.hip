@@ -1,0 +1,51 @@
+// Library-wide pieces of the C ABI: status strings, launch-error bookkeeping, device check.
+#include <string.h>
+
+#include "isp_common.h"
+
+namespace isp {
+
+static thread_local int t_last_hip_error = 0;
+
+int note_launch(hipError_t e) {
+    if (e == hipSuccess) return ISP_OK;
+    t_last_hip_error = (int)e;
+    return ISP_ERR_LAUNCH;
+}
+
+}  // namespace isp
+
+extern "C" {
+
+const char* isp_version(void) { return "inferspore_amd 0.1 (gfx950)"; }
+
+const char* isp_strerror(int status) {
+    switch (status) {
+        case ISP_OK: return "ok";
+        case ISP_ERR_NULL_POINTER: return "a required pointer is NULL";
+        case ISP_ERR_BAD_SHAPE: return "negative or inconsistent extents";
+        case ISP_ERR_UNSUPPORTED: return "extents outside what the kernels implement";
+        case ISP_ERR_LAUNCH: return "HIP reported an error at kernel launch";
+        case ISP_ERR_DEVICE: return "no usable gfx950 device";
+        default: return "unknown status";
+    }
+}
+
+int isp_last_hip_error(void) { return isp::t_last_hip_error; }
+
+int isp_init(void) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) {
+        (void)hipGetLastError();
+        return ISP_ERR_DEVICE;
+    }
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, dev) != hipSuccess) {
+        (void)hipGetLastError();
+        return ISP_ERR_DEVICE;
+    }
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0) return ISP_ERR_DEVICE;
+    return ISP_OK;
+}
+
+}  // extern "C"

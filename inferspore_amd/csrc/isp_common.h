@@ -1,0 +1,125 @@
+// Shared host/device helpers for the gfx950 kernels.
+#pragma once
+
+#include <hip/hip_fp16.h>
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "inferspore_amd.h"
+
+namespace isp {
+
+constexpr int kWave = 64;     // CDNA wavefront width
+constexpr int kBlock = 256;   // threads per workgroup used by every kernel here (4 waves)
+
+// ----------------------------------------------------------------------------- host side
+
+// Records a failed launch for isp_last_hip_error(); returns the status to hand back.
+int note_launch(hipError_t e);
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+#define ISP_REQUIRE_PTR(p)                   \
+    do {                                     \
+        if ((p) == nullptr) return ISP_ERR_NULL_POINTER; \
+    } while (0)
+
+// ----------------------------------------------------------------------------- device side
+
+// 16-byte vector used for every global access on the fast paths (global_load_dwordx4).
+struct __attribute__((aligned(16))) vec16 {
+    uint32_t w[4];
+};
+
+__device__ __forceinline__ vec16 load16(const void* p) {
+    return *reinterpret_cast<const vec16*>(p);
+}
+__device__ __forceinline__ void store16(void* p, const vec16& v) {
+    *reinterpret_cast<vec16*>(p) = v;
+}
+// Streaming variants: data touched once is marked non-temporal so it does not displace the small
+// operands (gamma, bias, tables) that every row re-reads.
+__device__ __forceinline__ vec16 load16_stream(const void* p) {
+    vec16 v;
+    const uint32_t* q = reinterpret_cast<const uint32_t*>(p);
+    typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+    u4 t = __builtin_nontemporal_load(reinterpret_cast<const u4*>(q));
+    v.w[0] = t.x; v.w[1] = t.y; v.w[2] = t.z; v.w[3] = t.w;
+    return v;
+}
+__device__ __forceinline__ void store16_stream(void* p, const vec16& v) {
+    typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+    u4 t = {v.w[0], v.w[1], v.w[2], v.w[3]};
+    __builtin_nontemporal_store(t, reinterpret_cast<u4*>(p));
+}
+
+// Element traits: how many elements a 16-byte vector holds and how to move between storage and fp32.
+template <typename T>
+struct Elem;
+
+template <>
+struct Elem<float> {
+    static constexpr int kVec = 4;
+    __device__ static __forceinline__ void unpack(const vec16& v, float* f) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) f[i] = __uint_as_float(v.w[i]);
+    }
+    __device__ static __forceinline__ vec16 pack(const float* f) {
+        vec16 v;
+#pragma unroll
+        for (int i = 0; i < 4; i++) v.w[i] = __float_as_uint(f[i]);
+        return v;
+    }
+    __device__ static __forceinline__ float to_f32(float x) { return x; }
+    __device__ static __forceinline__ float from_f32(float x) { return x; }
+};
+
+template <>
+struct Elem<__half> {
+    static constexpr int kVec = 8;
+    __device__ static __forceinline__ void unpack(const vec16& v, float* f) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            __half2 h = *reinterpret_cast<const __half2*>(&v.w[i]);
+            float2 p = __half22float2(h);
+            f[2 * i] = p.x;
+            f[2 * i + 1] = p.y;
+        }
+    }
+    __device__ static __forceinline__ vec16 pack(const float* f) {
+        vec16 v;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            __half2 h = __floats2half2_rn(f[2 * i], f[2 * i + 1]);
+            v.w[i] = *reinterpret_cast<const uint32_t*>(&h);
+        }
+        return v;
+    }
+    __device__ static __forceinline__ float to_f32(__half x) { return __half2float(x); }
+    __device__ static __forceinline__ __half from_f32(float x) { return __float2half_rn(x); }
+};
+
+// DPP lane exchange inside the VALU (no LDS traffic).  `ctrl` is the DPP control word.
+template <int ctrl>
+__device__ __forceinline__ float dpp_mov(float x) {
+    return __uint_as_float(
+        __builtin_amdgcn_update_dpp(0u, __float_as_uint(x), ctrl, 0xf, 0xf, true));
+}
+
+// Sum over the 64 lanes of a wavefront; every lane receives the total.
+// Four DPP steps fold each row of 16 lanes (quad swaps, then half-row and full-row mirrors), then
+// the four row sums are read out as scalars and added in a fixed order, so the result is
+// deterministic and identical in all lanes.
+__device__ __forceinline__ float wave_sum(float x) {
+    x += dpp_mov<0xB1>(x);   // quad_perm [1,0,3,2]
+    x += dpp_mov<0x4E>(x);   // quad_perm [2,3,0,1]
+    x += dpp_mov<0x141>(x);  // row_half_mirror
+    x += dpp_mov<0x140>(x);  // row_mirror
+    float a = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(x), 0));
+    float b = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(x), 16));
+    float c = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(x), 32));
+    float d = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(x), 48));
+    return (a + b) + (c + d);
+}
+
+}  // namespace isp

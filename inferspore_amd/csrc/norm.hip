@@ -1,0 +1,238 @@
+// RMSNorm and fused add-bias + residual + RMSNorm for gfx950.
+//
+// Semantics follow the reference's fp32 kernel (src/kernels/fused_addresidual_norm.cu:55-97):
+//   x = out + residual (+ bias);  residual := x;  out := gamma * x * rsqrt(sum(x^2)/H + eps)
+// with optional residual and bias.  Design (not the reference's): the whole row stays in fp32
+// registers between the sum of squares and the scaling, so every tensor crosses HBM exactly once
+// (the reference re-reads and read-modify-writes decoder_out); all global accesses are 16-byte
+// vectors; the row sum is a DPP wave reduction plus, when a row spans several waves, one small LDS
+// combine behind a single barrier.
+#include "isp_common.h"
+
+namespace isp {
+
+// One row is handled by WPR waves (ROW_THREADS = 64 * WPR lanes); a 256-thread workgroup therefore
+// carries 4 / WPR rows.  Each lane owns NV 16-byte vectors of the row, strided by ROW_THREADS so
+// that every load instruction of a wave covers 1 KiB of contiguous memory.
+template <typename T, int NV, int WPR>
+__global__ __launch_bounds__(kBlock) void fused_norm_rows(T* __restrict__ residual,
+                                                          T* __restrict__ out,
+                                                          const T* __restrict__ bias,
+                                                          const T* __restrict__ gamma, float eps,
+                                                          int tokens, int hidden, unsigned flags) {
+    constexpr int VEC = Elem<T>::kVec;
+    constexpr int ROW_THREADS = kWave * WPR;
+    constexpr int ROWS = kBlock / ROW_THREADS;
+
+    const int slot = threadIdx.x / ROW_THREADS;
+    const int lane = threadIdx.x % ROW_THREADS;
+    const int row = blockIdx.x * ROWS + slot;
+    const bool live = row < tokens;  // uniform within a wave
+    const int nvec = hidden / VEC;
+    const size_t base = (size_t)(live ? row : 0) * (size_t)hidden;
+    T* out_row = out + base;
+    T* rsd_row = residual ? residual + base : nullptr;
+
+    vec16 vo[NV], vr[NV];
+    bool ok[NV];
+#pragma unroll
+    for (int j = 0; j < NV; j++) {
+        const int vi = lane + j * ROW_THREADS;
+        ok[j] = live && vi < nvec;
+        if (ok[j]) {
+            vo[j] = load16_stream(out_row + (size_t)vi * VEC);
+            if (rsd_row) vr[j] = load16_stream(rsd_row + (size_t)vi * VEC);
+        }
+    }
+
+    float x[NV][VEC];
+    float acc = 0.0f;
+#pragma unroll
+    for (int j = 0; j < NV; j++) {
+        if (ok[j]) {
+            const int vi = lane + j * ROW_THREADS;
+            Elem<T>::unpack(vo[j], x[j]);
+            if (rsd_row) {
+                float r[VEC];
+                Elem<T>::unpack(vr[j], r);
+#pragma unroll
+                for (int e = 0; e < VEC; e++) x[j][e] += r[e];
+                if (flags & ISP_NORM_RESIDUAL_EXCLUDES_BIAS)
+                    store16(rsd_row + (size_t)vi * VEC, Elem<T>::pack(x[j]));
+            }
+            if (bias) {
+                float b[VEC];
+                Elem<T>::unpack(load16(bias + (size_t)vi * VEC), b);
+#pragma unroll
+                for (int e = 0; e < VEC; e++) x[j][e] += b[e];
+            }
+            if (rsd_row && !(flags & ISP_NORM_RESIDUAL_EXCLUDES_BIAS))
+                store16(rsd_row + (size_t)vi * VEC, Elem<T>::pack(x[j]));
+#pragma unroll
+            for (int e = 0; e < VEC; e++) acc += x[j][e] * x[j][e];
+        }
+    }
+
+    float total = wave_sum(acc);
+    if (WPR > 1) {
+        __shared__ float partial[kBlock / kWave];
+        const int wave = threadIdx.x / kWave;
+        if ((threadIdx.x % kWave) == 0) partial[wave] = total;
+        __syncthreads();
+        total = 0.0f;
+#pragma unroll
+        for (int w = 0; w < WPR; w++) total += partial[slot * WPR + w];
+    }
+    const float inv = rsqrtf(total / (float)hidden + eps);
+
+#pragma unroll
+    for (int j = 0; j < NV; j++) {
+        if (ok[j]) {
+            const int vi = lane + j * ROW_THREADS;
+            float g[VEC];
+            Elem<T>::unpack(load16(gamma + (size_t)vi * VEC), g);
+            float y[VEC];
+#pragma unroll
+            for (int e = 0; e < VEC; e++) y[e] = g[e] * x[j][e] * inv;
+            store16(out_row + (size_t)vi * VEC, Elem<T>::pack(y));
+        }
+    }
+}
+
+// Any hidden size and any alignment: one workgroup per row, scalar accesses, two passes over the
+// inputs (the first only accumulates, the second recomputes x with the same fp32 operations and
+// stores), so nothing is overwritten before it has been read for the last time.
+template <typename T>
+__global__ __launch_bounds__(kBlock) void fused_norm_generic(T* residual, T* out, const T* bias,
+                                                             const T* gamma, float eps, int tokens,
+                                                             int hidden, unsigned flags) {
+    const int row = blockIdx.x;
+    T* out_row = out + (size_t)row * hidden;
+    T* rsd_row = residual ? residual + (size_t)row * hidden : nullptr;
+    float acc = 0.0f;
+    for (int i = threadIdx.x; i < hidden; i += kBlock) {
+        float x = Elem<T>::to_f32(out_row[i]);
+        if (rsd_row) x += Elem<T>::to_f32(rsd_row[i]);
+        if (bias) x += Elem<T>::to_f32(bias[i]);
+        acc += x * x;
+    }
+    __shared__ float partial[kBlock / kWave];
+    float total = wave_sum(acc);
+    if ((threadIdx.x % kWave) == 0) partial[threadIdx.x / kWave] = total;
+    __syncthreads();
+    total = (partial[0] + partial[1]) + (partial[2] + partial[3]);
+    const float inv = rsqrtf(total / (float)hidden + eps);
+    for (int i = threadIdx.x; i < hidden; i += kBlock) {
+        float x = Elem<T>::to_f32(out_row[i]);
+        if (rsd_row) {
+            x += Elem<T>::to_f32(rsd_row[i]);
+            if (flags & ISP_NORM_RESIDUAL_EXCLUDES_BIAS) rsd_row[i] = Elem<T>::from_f32(x);
+        }
+        if (bias) x += Elem<T>::to_f32(bias[i]);
+        if (rsd_row && !(flags & ISP_NORM_RESIDUAL_EXCLUDES_BIAS)) rsd_row[i] = Elem<T>::from_f32(x);
+        out_row[i] = Elem<T>::from_f32(Elem<T>::to_f32(gamma[i]) * x * inv);
+    }
+}
+
+template <typename T, int NV, int WPR>
+static hipError_t launch_rows(T* residual, T* out, const T* bias, const T* gamma, float eps,
+                              int tokens, int hidden, unsigned flags, hipStream_t s) {
+    constexpr int ROWS = kBlock / (kWave * WPR);
+    dim3 grid((unsigned)((tokens + ROWS - 1) / ROWS));
+    hipLaunchKernelGGL((fused_norm_rows<T, NV, WPR>), grid, dim3(kBlock), 0, s, residual, out, bias,
+                       gamma, eps, tokens, hidden, flags);
+    return hipGetLastError();
+}
+
+template <typename T, int WPR>
+static hipError_t launch_rows_nv(int nv, T* residual, T* out, const T* bias, const T* gamma,
+                                 float eps, int tokens, int hidden, unsigned flags, hipStream_t s) {
+    if (nv <= 1) return launch_rows<T, 1, WPR>(residual, out, bias, gamma, eps, tokens, hidden, flags, s);
+    if (nv <= 2) return launch_rows<T, 2, WPR>(residual, out, bias, gamma, eps, tokens, hidden, flags, s);
+    if (nv <= 4) return launch_rows<T, 4, WPR>(residual, out, bias, gamma, eps, tokens, hidden, flags, s);
+    return launch_rows<T, 8, WPR>(residual, out, bias, gamma, eps, tokens, hidden, flags, s);
+}
+
+// Waves per row: rows per workgroup trade against loads in flight per lane.  tuning_wpr() lets the
+// benchmark sweep the choice (0 = automatic).
+static int g_norm_wpr = 0;
+
+template <typename T>
+static int fused_norm(void* residual_, void* out_, const void* bias_, const void* gamma_, float eps,
+                      int tokens, int hidden, unsigned flags, hipStream_t s) {
+    if (tokens < 0 || hidden < 0) return ISP_ERR_BAD_SHAPE;
+    if (tokens == 0 || hidden == 0) return ISP_OK;
+    ISP_REQUIRE_PTR(out_);
+    ISP_REQUIRE_PTR(gamma_);
+    T* residual = static_cast<T*>(residual_);
+    T* out = static_cast<T*>(out_);
+    const T* bias = static_cast<const T*>(bias_);
+    const T* gamma = static_cast<const T*>(gamma_);
+    constexpr int VEC = Elem<T>::kVec;
+    constexpr int MAX_NV = 8;
+
+    const bool vec_ok = (hidden % VEC == 0) && aligned16(out) && aligned16(gamma) &&
+                        (!residual || aligned16(residual)) && (!bias || aligned16(bias)) &&
+                        (hidden / VEC) <= MAX_NV * kBlock;
+    hipError_t e;
+    if (!vec_ok) {
+        hipLaunchKernelGGL((fused_norm_generic<T>), dim3((unsigned)tokens), dim3(kBlock), 0, s,
+                           residual, out, bias, gamma, eps, tokens, hidden, flags);
+        e = hipGetLastError();
+    } else {
+        const int nvec = hidden / VEC;
+        int wpr = g_norm_wpr;
+        if (wpr != 1 && wpr != 2 && wpr != 4) {
+            // automatic: the fewest waves per row that keep at most 4 vectors per lane in flight
+            wpr = 1;
+            while (wpr < 4 && (nvec + kWave * wpr - 1) / (kWave * wpr) > 4) wpr *= 2;
+        }
+        while (wpr < 4 && (nvec + kWave * wpr - 1) / (kWave * wpr) > MAX_NV) wpr *= 2;
+        const int nv = (nvec + kWave * wpr - 1) / (kWave * wpr);
+        if (wpr == 1)
+            e = launch_rows_nv<T, 1>(nv, residual, out, bias, gamma, eps, tokens, hidden, flags, s);
+        else if (wpr == 2)
+            e = launch_rows_nv<T, 2>(nv, residual, out, bias, gamma, eps, tokens, hidden, flags, s);
+        else
+            e = launch_rows_nv<T, 4>(nv, residual, out, bias, gamma, eps, tokens, hidden, flags, s);
+    }
+    return note_launch(e);
+}
+
+}  // namespace isp
+
+extern "C" {
+
+int isp_tuning_norm_waves_per_row(int wpr) {
+    int old = isp::g_norm_wpr;
+    isp::g_norm_wpr = wpr;
+    return old;
+}
+
+int isp_fused_add_bias_residual_rmsnorm_f32(void* residual, void* decoder_out, const void* bias,
+                                            const void* gamma, float eps, int tokens, int hidden,
+                                            unsigned flags, isp_stream_t stream) {
+    return isp::fused_norm<float>(residual, decoder_out, bias, gamma, eps, tokens, hidden, flags,
+                                  static_cast<hipStream_t>(stream));
+}
+
+int isp_fused_add_bias_residual_rmsnorm_f16(void* residual, void* decoder_out, const void* bias,
+                                            const void* gamma, float eps, int tokens, int hidden,
+                                            unsigned flags, isp_stream_t stream) {
+    return isp::fused_norm<__half>(residual, decoder_out, bias, gamma, eps, tokens, hidden, flags,
+                                   static_cast<hipStream_t>(stream));
+}
+
+int isp_rmsnorm_f32(void* x, const void* gamma, float eps, int tokens, int hidden,
+                    isp_stream_t stream) {
+    return isp::fused_norm<float>(nullptr, x, nullptr, gamma, eps, tokens, hidden, 0u,
+                                  static_cast<hipStream_t>(stream));
+}
+
+int isp_rmsnorm_f16(void* x, const void* gamma, float eps, int tokens, int hidden,
+                    isp_stream_t stream) {
+    return isp::fused_norm<__half>(nullptr, x, nullptr, gamma, eps, tokens, hidden, 0u,
+                                   static_cast<hipStream_t>(stream));
+}
+
+}  // extern "C"

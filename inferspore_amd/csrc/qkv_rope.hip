@@ -1,0 +1,274 @@
+// Fused QKV bias + rotate-half RoPE + head transpose + re-padding (prefill) for gfx950.
+//
+// Semantics: src/kernels/qkv_bias_and_RoPE.cu:132-191 (fp32 kernel) with the bias indexing of that
+// file's disabled fp16 body (:239,247,250):
+//   p = token + padding_offset[token];  b = p / seq_len;  s = p % seq_len;  t = history[b] + s
+//   x = qkv[token, head, d] (+ bias[head, d])
+//   q/k heads, d < rot/2:  angle = t / base^(2d/rot)
+//       out[d]        = cos * x[d]        - sin * x[d + hs/2]
+//       out[d + hs/2] = cos * x[d + hs/2] + sin * x[d]
+//   v heads and un-rotated elements are copied;  destination [b, head, s, :] of q / k / v.
+//
+// Design (not the reference's one-thread-per-element, one-block-per-(token, head) kernel):
+//   * one 256-thread workgroup per token; the 64 distinct (cos, sin) pairs of that token are
+//     evaluated once by 64 lanes, parked in 512 bytes of LDS and reused by all q and k heads (the
+//     reference evaluates powf + cos + sin again for every head);
+//   * the divisors base^(2d/rot) do not depend on the data, so the host computes them once per
+//     launch configuration with the C library's powf and passes them by value in the kernel
+//     arguments: the device forms angle = t / divisor with one correctly rounded division;
+//   * a lane owns 16 bytes at d = VEC*g and the 16 bytes of the rotation partners at d + hs/2, so
+//     the rotate-half pairing needs no cross-lane exchange, and each group of hs/(2 VEC) lanes
+//     reads and writes whole 128-byte lines of one head row;
+//   * each lane keeps up to UNROLL heads (2 UNROLL vector loads) in flight before computing.
+#include <math.h>
+
+#include "isp_common.h"
+
+namespace isp {
+
+constexpr int kMaxHalfRot = 128;  // rotary_embedding_dim up to 256
+
+struct RopeDivisors {
+    float div[kMaxHalfRot];
+};
+
+template <typename T, int HS, int UNROLL>
+__global__ __launch_bounds__(kBlock) void qkv_rope_vec(
+    T* __restrict__ q, T* __restrict__ k, T* __restrict__ v, const T* __restrict__ qkv,
+    const T* __restrict__ bias, const int32_t* __restrict__ padding_offset,
+    const int32_t* __restrict__ history_length, int batch, int seq_len, int head_num,
+    int kv_head_num, int half_rot, RopeDivisors tab) {
+    constexpr int VEC = Elem<T>::kVec;
+    constexpr int HALF = HS / 2;
+    constexpr int G = HALF / VEC;  // lanes per head
+    static_assert(HALF % VEC == 0 && kWave % G == 0, "head size must split into whole lanes");
+    constexpr int HEADS_PER_WAVE = kWave / G;
+    constexpr int HEADS_PER_PASS = HEADS_PER_WAVE * (kBlock / kWave);
+
+    const int token = blockIdx.x;
+    const long long p = (long long)token + (long long)padding_offset[token];
+    if (p < 0 || p >= (long long)batch * (long long)seq_len) return;  // uniform: whole block leaves
+    const int b = (int)(p / seq_len);
+    const int s = (int)(p % seq_len);
+    const int timestep = history_length[b] + s;
+
+    __shared__ float2 cs[HALF];
+    if (threadIdx.x < HALF) {
+        float c = 1.0f, sn = 0.0f;
+        if ((int)threadIdx.x < half_rot) {
+            const float angle = (float)timestep / tab.div[threadIdx.x];
+            sincosf(angle, &sn, &c);
+        }
+        cs[threadIdx.x] = make_float2(c, sn);
+    }
+    __syncthreads();
+
+    const int lane = threadIdx.x % kWave;
+    const int wave = threadIdx.x / kWave;
+    const int g = lane % G;
+    const int slot = lane / G;
+    float c[VEC], sn[VEC];
+    bool rot[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; e++) {
+        const float2 t = cs[g * VEC + e];
+        c[e] = t.x;
+        sn[e] = t.y;
+        rot[e] = (g * VEC + e) < half_rot;
+    }
+
+    const int qkv_heads = head_num + 2 * kv_head_num;
+    const T* row = qkv + (size_t)token * (size_t)qkv_heads * HS;
+    const int col = g * VEC;
+
+    for (int h0 = wave * HEADS_PER_WAVE + slot; h0 < qkv_heads; h0 += HEADS_PER_PASS * UNROLL) {
+        vec16 lo[UNROLL], hi[UNROLL];
+#pragma unroll
+        for (int u = 0; u < UNROLL; u++) {
+            const int h = h0 + u * HEADS_PER_PASS;
+            if (h < qkv_heads) {
+                lo[u] = load16_stream(row + (size_t)h * HS + col);
+                hi[u] = load16_stream(row + (size_t)h * HS + HALF + col);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < UNROLL; u++) {
+            const int h = h0 + u * HEADS_PER_PASS;
+            if (h < qkv_heads) {
+                float x0[VEC], x1[VEC];
+                Elem<T>::unpack(lo[u], x0);
+                Elem<T>::unpack(hi[u], x1);
+                if (bias) {
+                    float b0[VEC], b1[VEC];
+                    Elem<T>::unpack(load16(bias + (size_t)h * HS + col), b0);
+                    Elem<T>::unpack(load16(bias + (size_t)h * HS + HALF + col), b1);
+#pragma unroll
+                    for (int e = 0; e < VEC; e++) {
+                        x0[e] += b0[e];
+                        x1[e] += b1[e];
+                    }
+                }
+                T* dst;
+                bool rotate = true;
+                if (h < head_num) {
+                    dst = q + (((size_t)b * head_num + h) * seq_len + s) * HS;
+                } else if (h < head_num + kv_head_num) {
+                    dst = k + (((size_t)b * kv_head_num + (h - head_num)) * seq_len + s) * HS;
+                } else {
+                    dst = v + (((size_t)b * kv_head_num + (h - head_num - kv_head_num)) * seq_len + s) * HS;
+                    rotate = false;
+                }
+                float y0[VEC], y1[VEC];
+#pragma unroll
+                for (int e = 0; e < VEC; e++) {
+                    const bool r = rotate && rot[e];
+                    y0[e] = r ? c[e] * x0[e] - sn[e] * x1[e] : x0[e];
+                    y1[e] = r ? c[e] * x1[e] + sn[e] * x0[e] : x1[e];
+                }
+                store16(dst + col, Elem<T>::pack(y0));
+                store16(dst + HALF + col, Elem<T>::pack(y1));
+            }
+        }
+    }
+}
+
+// Any (even) head size and any alignment: one workgroup per token, one lane per rotation pair.
+template <typename T>
+__global__ __launch_bounds__(kBlock) void qkv_rope_generic(
+    T* q, T* k, T* v, const T* qkv, const T* bias, const int32_t* padding_offset,
+    const int32_t* history_length, int batch, int seq_len, int head_num, int kv_head_num,
+    int head_size, int half_rot, RopeDivisors tab) {
+    const int token = blockIdx.x;
+    const long long p = (long long)token + (long long)padding_offset[token];
+    if (p < 0 || p >= (long long)batch * (long long)seq_len) return;
+    const int b = (int)(p / seq_len);
+    const int s = (int)(p % seq_len);
+    const int timestep = history_length[b] + s;
+    const int half = head_size / 2;
+    const int qkv_heads = head_num + 2 * kv_head_num;
+    const T* row = qkv + (size_t)token * (size_t)qkv_heads * head_size;
+    const int pairs = qkv_heads * half;
+    for (int i = threadIdx.x; i < pairs; i += kBlock) {
+        const int h = i / half;
+        const int d = i % half;
+        float x0 = Elem<T>::to_f32(row[(size_t)h * head_size + d]);
+        float x1 = Elem<T>::to_f32(row[(size_t)h * head_size + half + d]);
+        if (bias) {
+            x0 += Elem<T>::to_f32(bias[(size_t)h * head_size + d]);
+            x1 += Elem<T>::to_f32(bias[(size_t)h * head_size + half + d]);
+        }
+        T* dst;
+        bool rotate = d < half_rot;
+        if (h < head_num) {
+            dst = q + (((size_t)b * head_num + h) * seq_len + s) * head_size;
+        } else if (h < head_num + kv_head_num) {
+            dst = k + (((size_t)b * kv_head_num + (h - head_num)) * seq_len + s) * head_size;
+        } else {
+            dst = v + (((size_t)b * kv_head_num + (h - head_num - kv_head_num)) * seq_len + s) * head_size;
+            rotate = false;
+        }
+        float y0 = x0, y1 = x1;
+        if (rotate) {
+            float c, sn;
+            sincosf((float)timestep / tab.div[d], &sn, &c);
+            y0 = c * x0 - sn * x1;
+            y1 = c * x1 + sn * x0;
+        }
+        dst[d] = Elem<T>::from_f32(y0);
+        dst[half + d] = Elem<T>::from_f32(y1);
+    }
+}
+
+template <typename T>
+static int qkv_rope(void* q_, void* k_, void* v_, const void* qkv_, const void* bias_,
+                    const int32_t* padding_offset, const int32_t* history_length,
+                    const int32_t* input_length, int batch, int seq_len, int token_num,
+                    int head_num, int kv_head_num, int head_size, int rot, float base,
+                    hipStream_t s) {
+    (void)input_length;  // read by the reference kernel, result unused (qkv_bias_and_RoPE.cu:161)
+    if (batch < 0 || seq_len < 0 || token_num < 0 || head_num < 0 || kv_head_num < 0 ||
+        head_size < 0 || rot < 0)
+        return ISP_ERR_BAD_SHAPE;
+    if (token_num == 0 || head_size == 0 || head_num + kv_head_num == 0) return ISP_OK;
+    if (batch == 0 || seq_len == 0) return ISP_ERR_BAD_SHAPE;
+    if (head_size % 2 != 0 || rot % 2 != 0 || rot > head_size) return ISP_ERR_BAD_SHAPE;
+    if (rot / 2 > kMaxHalfRot) return ISP_ERR_UNSUPPORTED;
+    if ((long long)head_num + 2ll * kv_head_num > 0x7fffffffll / (head_size > 0 ? head_size : 1))
+        return ISP_ERR_UNSUPPORTED;
+    ISP_REQUIRE_PTR(qkv_);
+    ISP_REQUIRE_PTR(padding_offset);
+    ISP_REQUIRE_PTR(history_length);
+    if (head_num > 0) ISP_REQUIRE_PTR(q_);
+    if (kv_head_num > 0) {
+        ISP_REQUIRE_PTR(k_);
+        ISP_REQUIRE_PTR(v_);
+    }
+    T* q = static_cast<T*>(q_);
+    T* k = static_cast<T*>(k_);
+    T* v = static_cast<T*>(v_);
+    const T* qkv = static_cast<const T*>(qkv_);
+    const T* bias = static_cast<const T*>(bias_);
+
+    RopeDivisors tab;
+    const int half_rot = rot / 2;
+    for (int d = 0; d < kMaxHalfRot; d++)
+        tab.div[d] = d < half_rot ? powf(base, (float)(2 * d) / (float)rot) : 1.0f;
+
+    const bool vec_ok = aligned16(q) && aligned16(k) && aligned16(v) && aligned16(qkv) &&
+                        (!bias || aligned16(bias));
+    dim3 grid((unsigned)token_num), block(kBlock);
+    hipError_t e;
+    if (vec_ok && head_size == 128) {
+        hipLaunchKernelGGL((qkv_rope_vec<T, 128, 4>), grid, block, 0, s, q, k, v, qkv, bias,
+                           padding_offset, history_length, batch, seq_len, head_num, kv_head_num,
+                           half_rot, tab);
+        e = hipGetLastError();
+    } else if (vec_ok && head_size == 64) {
+        hipLaunchKernelGGL((qkv_rope_vec<T, 64, 4>), grid, block, 0, s, q, k, v, qkv, bias,
+                           padding_offset, history_length, batch, seq_len, head_num, kv_head_num,
+                           half_rot, tab);
+        e = hipGetLastError();
+    } else {
+        hipLaunchKernelGGL((qkv_rope_generic<T>), grid, block, 0, s, q, k, v, qkv, bias,
+                           padding_offset, history_length, batch, seq_len, head_num, kv_head_num,
+                           head_size, half_rot, tab);
+        e = hipGetLastError();
+    }
+    return note_launch(e);
+}
+
+}  // namespace isp
+
+extern "C" {
+
+int isp_qkv_bias_rope_transpose_f32(void* q, void* k, void* v, const void* qkv, const void* bias,
+                                    const int32_t* padding_offset, const int32_t* history_length,
+                                    const int32_t* input_length, int batch, int seq_len,
+                                    int token_num, int head_num, int kv_head_num, int head_size,
+                                    int rotary_embedding_dim, float rotary_embedding_base,
+                                    int max_position_embeddings, int use_dynamic_ntk,
+                                    isp_stream_t stream) {
+    (void)max_position_embeddings;
+    (void)use_dynamic_ntk;
+    return isp::qkv_rope<float>(q, k, v, qkv, bias, padding_offset, history_length, input_length,
+                                batch, seq_len, token_num, head_num, kv_head_num, head_size,
+                                rotary_embedding_dim, rotary_embedding_base,
+                                static_cast<hipStream_t>(stream));
+}
+
+int isp_qkv_bias_rope_transpose_f16(void* q, void* k, void* v, const void* qkv, const void* bias,
+                                    const int32_t* padding_offset, const int32_t* history_length,
+                                    const int32_t* input_length, int batch, int seq_len,
+                                    int token_num, int head_num, int kv_head_num, int head_size,
+                                    int rotary_embedding_dim, float rotary_embedding_base,
+                                    int max_position_embeddings, int use_dynamic_ntk,
+                                    isp_stream_t stream) {
+    (void)max_position_embeddings;
+    (void)use_dynamic_ntk;
+    return isp::qkv_rope<__half>(q, k, v, qkv, bias, padding_offset, history_length, input_length,
+                                 batch, seq_len, token_num, head_num, kv_head_num, head_size,
+                                 rotary_embedding_dim, rotary_embedding_base,
+                                 static_cast<hipStream_t>(stream));
+}
+
+}  // extern "C"

@@ -1,0 +1,85 @@
+"""Host-side checks that need no GPU: the C-ABI library loads, exports every function its public
+header declares, and rejects bad arguments before touching the device."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_functions():
+    text = open(os.path.join(ROOT, "include", "inferspore_amd.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(isp_[a-z0-9_]+)\s*\(", text)))
+
+
+@pytest.fixture(scope="module")
+def lib():
+    from inferspore_amd import capi
+    return capi.lib()
+
+
+def test_header_declares_the_expected_entry_points():
+    names = declared_functions()
+    for n in ("isp_embedding_f16", "isp_rmsnorm_f32", "isp_fused_add_bias_residual_rmsnorm_f16",
+              "isp_qkv_bias_rope_transpose_f16", "isp_swiglu_f16", "isp_cal_padding_offset"):
+        assert n in names
+
+
+def test_library_exports_every_declared_symbol(lib):
+    from inferspore_amd import capi
+    for name in declared_functions():
+        assert hasattr(lib, name), "libinferspore_amd.so does not export " + name
+        assert name in capi.SIGNATURES, "no ctypes signature for " + name
+
+
+def test_version_and_error_strings(lib):
+    assert b"gfx950" in lib.isp_version()
+    for code in (0, -1, -2, -3, -4, -5):
+        assert lib.isp_strerror(code)
+    assert lib.isp_strerror(-99) == b"unknown status"
+
+
+def test_argument_validation_returns_before_any_launch(lib):
+    from inferspore_amd import capi
+    p = ctypes.c_void_p(16)  # a non-NULL placeholder; validation fails before it is dereferenced
+    # zero work is OK whatever the pointers are
+    assert lib.isp_swiglu_f16(None, None, 0, 11008, None) == capi.OK
+    assert lib.isp_embedding_f16(None, None, None, 0, 4096, 0, None) == capi.OK
+    assert lib.isp_rmsnorm_f32(None, None, 1e-5, 0, 4096, None) == capi.OK
+    # NULL required operands
+    assert lib.isp_swiglu_f16(None, p, 4, 8, None) == capi.ERR_NULL_POINTER
+    assert lib.isp_embedding_f32(p, None, p, 4, 8, 0, None) == capi.ERR_NULL_POINTER
+    assert lib.isp_rmsnorm_f16(p, None, 1e-5, 4, 8, None) == capi.ERR_NULL_POINTER
+    assert lib.isp_fused_add_bias_residual_rmsnorm_f16(None, None, None, p, 1e-5, 4, 8, 0, None) == capi.ERR_NULL_POINTER
+    assert lib.isp_cal_padding_offset(p, None, p, 2, 4, None) == capi.ERR_NULL_POINTER
+    # negative extents
+    assert lib.isp_swiglu_f32(p, p, -1, 8, None) == capi.ERR_BAD_SHAPE
+    assert lib.isp_embedding_f16(p, p, p, 4, -8, 0, None) == capi.ERR_BAD_SHAPE
+    assert lib.isp_rmsnorm_f32(p, p, 1e-5, -4, 8, None) == capi.ERR_BAD_SHAPE
+    assert lib.isp_cal_padding_offset(p, p, p, -2, 4, None) == capi.ERR_BAD_SHAPE
+    qkv = lib.isp_qkv_bias_rope_transpose_f16
+    args = dict(batch=1, seq=4, tok=3, hn=2, kvn=2, hs=128, rot=128)
+
+    def call(q=p, k=p, v=p, x=p, po=p, hist=p, **kw):
+        a = dict(args, **kw)
+        return qkv(q, k, v, x, None, po, hist, p, a["batch"], a["seq"], a["tok"], a["hn"], a["kvn"], a["hs"],
+                   a["rot"], 10000.0, 2048, 0, None)
+
+    assert call(tok=0) == capi.OK
+    assert call(x=None) == capi.ERR_NULL_POINTER
+    assert call(po=None) == capi.ERR_NULL_POINTER
+    assert call(q=None) == capi.ERR_NULL_POINTER
+    assert call(hs=127) == capi.ERR_BAD_SHAPE          # odd head size cannot be split in halves
+    assert call(rot=130) == capi.ERR_BAD_SHAPE         # rotary dim larger than the head
+    assert call(seq=0) == capi.ERR_BAD_SHAPE
+    assert call(hs=1024, rot=1024) == capi.ERR_UNSUPPORTED
+
+
+def test_python_layer_refuses_cpu_tensors():
+    import torch
+    from inferspore_amd import ops
+    with pytest.raises(RuntimeError, match="GPU"):
+        ops.act(torch.ones((2, 2, 8)), torch.empty((2, 8)))

@@ -1,0 +1,330 @@
+"""Parity of the HIP kernels (called through the C ABI) against the CPU oracle, on identical seeded
+inputs: the benchmark configurations at full size plus ragged / odd / empty cases that force every
+kernel variant (vector fast paths and scalar fallbacks)."""
+import numpy as np
+import pytest
+import torch
+
+from helpers import (assert_f16_close, assert_f32_close, embedding_inputs, norm_inputs, padding_offsets_np,
+                     qkv_inputs, swiglu_inputs)
+
+pytestmark = pytest.mark.gpu
+
+NP2T = {np.float16: torch.float16, np.float32: torch.float32}
+
+
+def dev(a):
+    return None if a is None else torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def host(t):
+    return t.cpu().numpy()
+
+
+def say(msg):
+    print("[case] " + msg, flush=True)
+
+
+# ------------------------------------------------------------------ embedding (bit-exact)
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+@pytest.mark.parametrize("tokens,hidden,vocab", [(8192, 4096, 32000), (64, 4096, 32000), (1, 8, 3), (37, 136, 513),
+                                                 (5, 7, 11), (300, 1000, 50)])
+def test_embedding(isp, oracle, dtype, tokens, hidden, vocab):
+    if dtype == np.float32 and vocab == 32000 and tokens == 8192:
+        vocab = 8000  # keep the fp32 table at 131 MB; the fp16 case is the benchmark configuration
+    say("embedding %s tokens=%d hidden=%d vocab=%d" % (dtype.__name__, tokens, hidden, vocab))
+    ids, table = embedding_inputs(tokens, hidden, vocab, dtype)
+    out = torch.full((tokens, hidden), 7, dtype=NP2T[dtype], device="cuda")
+    isp.input_embedding(dev(ids), out, dev(table))
+    torch.cuda.synchronize()
+    assert np.array_equal(host(out).view(np.uint8), oracle.embedding(ids, table).view(np.uint8))
+
+
+def test_embedding_known_answer_rows(isp):
+    # the reference's own check: table[r, :] = r  =>  out[t, :] = ids[t]
+    vocab, hidden, tokens = 32000, 4096, 64
+    table = torch.arange(vocab, dtype=torch.float32, device="cuda").to(torch.float16)[:, None].expand(vocab, hidden).contiguous()
+    ids = torch.from_numpy(np.random.default_rng(3).integers(0, vocab, tokens, dtype=np.int32)).cuda()
+    out = torch.empty((tokens, hidden), dtype=torch.float16, device="cuda")
+    isp.input_embedding(ids, out, table)
+    assert torch.equal(out, ids.to(torch.float32).to(torch.float16)[:, None].expand(tokens, hidden))
+
+
+def test_embedding_misaligned_and_bounds(isp, oracle):
+    ids, table = embedding_inputs(33, 24, 40, np.float16, seed=2)
+    big = torch.zeros(33 * 24 + 8, dtype=torch.float16, device="cuda")
+    out = big[1:1 + 33 * 24].view(33, 24)  # 2-byte aligned only: byte-copy kernel
+    isp.input_embedding(dev(ids), out, dev(table))
+    assert np.array_equal(host(out), oracle.embedding(ids, table))
+    # ids outside the table give zero rows when the vocabulary size is known
+    bad = ids.copy()
+    bad[[0, 5]] = [40, -1]
+    out2 = torch.full((33, 24), 3, dtype=torch.float16, device="cuda")
+    isp.input_embedding(dev(bad), out2, dev(table))
+    exp = oracle.embedding(np.where((bad < 0) | (bad >= 40), 0, bad), table)
+    exp[[0, 5]] = 0
+    assert np.array_equal(host(out2), exp)
+    # empty input is a no-op
+    isp.input_embedding(torch.empty(0, dtype=torch.int32, device="cuda"),
+                        torch.empty((0, 24), dtype=torch.float16, device="cuda"), dev(table))
+    with pytest.raises(RuntimeError):
+        isp.input_embedding(dev(ids[:5]), out2, dev(table))
+
+
+# ------------------------------------------------------------------ padding offset (bit-exact)
+@pytest.mark.parametrize("lens,max_q", [([3, 3, 3], 5), ([3, 2, 5], 5), ([1], 1), ([0, 4, 0, 2], 4), ([7] * 9, 7),
+                                        ("rand8", 512), ("rand700", 64)])
+def test_padding_offset(isp, oracle, lens, max_q):
+    if isinstance(lens, str):
+        n = int(lens[4:])
+        lens = np.random.default_rng(n).integers(max_q // 2, max_q + 1, n)
+    lens = np.asarray(lens, np.int32)
+    say("padding offset batch=%d max_q=%d" % (len(lens), max_q))
+    po = torch.full((len(lens), max_q), -5, dtype=torch.int32, device="cuda")
+    cum = torch.full((len(lens) + 1,), -5, dtype=torch.int32, device="cuda")
+    isp.cal_padding_offset(po, cum, dev(lens))
+    epo, ecum = oracle.cal_padding_offset(lens, max_q, fill=-5)
+    assert np.array_equal(host(po), epo)      # including the untouched tail
+    assert np.array_equal(host(cum), ecum)
+    npo, ncum = padding_offsets_np(lens, max_q)
+    assert np.array_equal(host(po).reshape(-1)[:len(npo)], npo) and np.array_equal(host(cum), ncum)
+
+
+def test_padding_offset_shape_checks(isp):
+    po = torch.zeros((3, 5), dtype=torch.int32, device="cuda")
+    with pytest.raises(RuntimeError):
+        isp.cal_padding_offset(po, torch.zeros(4, dtype=torch.int32, device="cuda"),
+                               torch.zeros(2, dtype=torch.int32, device="cuda"))
+    with pytest.raises(RuntimeError):
+        isp.cal_padding_offset(po, torch.zeros(3, dtype=torch.int32, device="cuda"),
+                               torch.zeros(3, dtype=torch.int32, device="cuda"))
+
+
+# ------------------------------------------------------------------ RMSNorm / fused norm
+def _check_norm(isp, oracle, dtype, tokens, hidden, with_res, with_bias, flags=0, wpr=0, seed=0):
+    from inferspore_amd import capi
+    res, out, bias, gamma = norm_inputs(tokens, hidden, dtype, seed=seed, with_residual=with_res, with_bias=with_bias)
+    d_res, d_out = dev(res), dev(out)
+    capi.lib().isp_tuning_norm_waves_per_row(wpr)
+    try:
+        isp.fused_add_bias_residual_rmsnorm(d_res, d_out, dev(bias), dev(gamma), 1e-5, flags=flags)
+        torch.cuda.synchronize()
+    finally:
+        capi.lib().isp_tuning_norm_waves_per_row(0)
+    e_res, e_out = oracle.fused_norm(res, out, bias, gamma, 1e-5, flags=flags)
+    if dtype == np.float32:
+        assert_f32_close(host(d_out), e_out, "normalised output")
+        if with_res:
+            assert np.array_equal(host(d_res), e_res), "residual must be the exact fp32 sum"
+    else:
+        assert_f16_close(host(d_out), e_out, "normalised output")
+        if with_res:
+            assert np.array_equal(host(d_res), e_res), "residual must be the once-rounded fp32 sum"
+
+
+def test_rmsnorm_config_fp32_64x4096(isp, oracle):
+    _, x, _, gamma = norm_inputs(64, 4096, np.float32, with_residual=False, with_bias=False)
+    d = dev(x)
+    isp.rmsnorm(d, dev(gamma), 1e-5)
+    e = oracle.rmsnorm(x, gamma, 1e-5)
+    assert_f32_close(host(d), e, "rmsnorm 64x4096 fp32")
+    x64 = x.astype(np.float64)
+    closed = x64 / np.sqrt((x64 * x64).mean(1, keepdims=True) + 1e-5) * gamma
+    assert_f32_close(host(d), closed, "rmsnorm vs closed form")
+
+
+def test_fused_norm_config_fp16_2048x4096(isp, oracle):
+    _check_norm(isp, oracle, np.float16, 2048, 4096, True, True)
+
+
+def test_fused_norm_known_answer(isp):
+    # reference test: out = 1, residual = 0, gamma = 1, eps = 0.5, H = 32  =>  1 / sqrt(1.5)
+    out = torch.ones((2, 32), device="cuda")
+    res = torch.zeros((2, 32), device="cuda")
+    isp.fused_add_bias_residual_rmsnorm(res, out, None, torch.ones(32, device="cuda"), 0.5)
+    assert torch.allclose(out, torch.full_like(out, 0.816496580927726), rtol=1e-6, atol=0)
+    assert torch.equal(res, torch.ones_like(res))
+
+
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+@pytest.mark.parametrize("wpr", [0, 1, 2, 4])
+@pytest.mark.parametrize("tokens,hidden", [(2048, 4096), (7, 4096), (1, 8), (13, 1000), (5, 8192), (3, 11008),
+                                           (2, 16384), (9, 520)])
+def test_fused_norm_variants(isp, oracle, dtype, wpr, tokens, hidden):
+    if tokens == 2048 and dtype == np.float32 and wpr not in (0, 4):
+        pytest.skip("covered by the fp16 sweep")
+    say("fused norm %s %dx%d wpr=%d" % (dtype.__name__, tokens, hidden, wpr))
+    _check_norm(isp, oracle, dtype, tokens, hidden, True, True, wpr=wpr, seed=tokens + hidden)
+
+
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+@pytest.mark.parametrize("with_res,with_bias,flags", [(True, False, 0), (False, True, 0), (False, False, 0),
+                                                      (True, True, 1), (True, False, 1)])
+def test_fused_norm_optional_operands(isp, oracle, dtype, with_res, with_bias, flags):
+    _check_norm(isp, oracle, dtype, 33, 4096, with_res, with_bias, flags=flags, seed=5)
+
+
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+@pytest.mark.parametrize("tokens,hidden", [(5, 7), (4, 4097), (3, 30), (2, 20000), (1, 1)])
+def test_fused_norm_scalar_fallback(isp, oracle, dtype, tokens, hidden):
+    say("fused norm generic %s %dx%d" % (dtype.__name__, tokens, hidden))
+    _check_norm(isp, oracle, dtype, tokens, hidden, True, True, seed=9)
+    _check_norm(isp, oracle, dtype, tokens, hidden, False, False, seed=9)
+
+
+def test_fused_norm_deterministic_and_empty(isp):
+    res, out, bias, gamma = norm_inputs(256, 4096, np.float16, seed=4)
+    outs = []
+    for _ in range(3):
+        d_res, d_out = dev(res), dev(out)
+        isp.fused_add_bias_residual_rmsnorm(d_res, d_out, dev(bias), dev(gamma), 1e-5)
+        outs.append((host(d_res), host(d_out)))
+    assert all(np.array_equal(o[0], outs[0][0]) and np.array_equal(o[1], outs[0][1]) for o in outs)
+    isp.fused_add_bias_residual_rmsnorm(None, torch.empty((0, 4096), dtype=torch.float16, device="cuda"), None,
+                                        dev(gamma), 1e-5)
+
+
+# ------------------------------------------------------------------ SwiGLU
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+@pytest.mark.parametrize("tokens,inter", [(256, 11008), (16, 11008), (1, 8), (3, 1000), (7, 13), (5, 11009), (1024, 11008)])
+def test_swiglu(isp, oracle, dtype, tokens, inter):
+    say("swiglu %s %dx%d" % (dtype.__name__, tokens, inter))
+    x = swiglu_inputs(tokens, inter, dtype, seed=tokens)
+    out = torch.full((tokens, inter), 9, dtype=NP2T[dtype], device="cuda")
+    isp.act(dev(x), out)
+    e = oracle.swiglu(x)
+    if dtype == np.float32:
+        assert_f32_close(host(out), e, "swiglu", scale=np.abs(e) + 1e-2 * np.abs(x[:, 1]))
+    else:
+        assert_f16_close(host(out), e, "swiglu")
+
+
+def test_swiglu_config_prefill_8192x11008_fp16(isp, oracle):
+    x = swiglu_inputs(8192, 11008, np.float16)
+    out = torch.empty((8192, 11008), dtype=torch.float16, device="cuda")
+    isp.act(dev(x), out)
+    got = host(out)
+    oracle.set_threads(16)
+    try:
+        e = oracle.swiglu(x)
+    finally:
+        oracle.set_threads(1)
+    assert_f16_close(got, e, "swiglu prefill")
+
+
+def test_swiglu_known_answer_and_special_values(isp):
+    x = torch.ones((16, 2, 11008), device="cuda")
+    out = torch.empty((16, 11008), device="cuda")
+    isp.act(x, out)
+    assert torch.allclose(out, torch.full_like(out, 0.7310585786300049), rtol=1e-6, atol=0)
+    out16 = torch.empty((16, 11008), dtype=torch.float16, device="cuda")
+    isp.act(x.half(), out16)
+    assert torch.all(out16 == 0.73095703125)
+    g = torch.tensor([0.0, -0.0, 20.0, -20.0, 65504.0, -65504.0, 11.0, -11.0], dtype=torch.float16, device="cuda")
+    x = torch.stack([g, torch.ones_like(g)])[None].contiguous()
+    o = torch.empty((1, 8), dtype=torch.float16, device="cuda")
+    isp.act(x, o)
+    o = o.float().cpu().numpy()[0]
+    assert np.isfinite(o).all() and o[0] == 0 and o[1] == 0 and o[4] == 65504.0 and o[5] == 0.0
+    assert abs((o[2] - o[3]) - 20.0) < 0.02 and abs((o[6] - o[7]) - 11.0) < 0.01
+    with pytest.raises(RuntimeError):
+        isp.act(torch.ones((4, 3, 8), device="cuda"), torch.empty((4, 8), device="cuda"))
+
+
+# ------------------------------------------------------------------ QKV bias + RoPE + transpose + re-pad
+def _check_qkv(isp, oracle, dtype, batch, seq, hn, kvn, hs, rot, with_bias=True, seed=0, min_len=None,
+               history=None, base=10000.0):
+    lens, qkv, bias, po, hist = qkv_inputs(batch, seq, hn, kvn, hs, dtype, seed=seed, min_len=min_len,
+                                           with_bias=with_bias)
+    if history is not None:
+        hist = np.asarray(history, np.int32)
+    td = NP2T[dtype]
+    sentinel = -77.0
+    q = torch.full((batch, hn, seq, hs), sentinel, dtype=td, device="cuda")
+    k = torch.full((batch, kvn, seq, hs), sentinel, dtype=td, device="cuda")
+    v = torch.full((batch, kvn, seq, hs), sentinel, dtype=td, device="cuda")
+    tokens = qkv.shape[0]
+    po_dev = torch.zeros((batch, seq), dtype=torch.int32, device="cuda")
+    po_dev.view(-1)[:tokens] = dev(po)
+    isp.add_fused_qkv_bias_transpose_and_rope(q, k, v, dev(qkv), dev(bias), po_dev, dev(hist), dev(lens), rot, base)
+    torch.cuda.synchronize()
+    eq, ek, ev = oracle.qkv_rope(qkv, bias, po, hist, lens, batch, seq, hn, kvn, rot, base, fill=sentinel)
+    gq, gk, gv = host(q), host(k), host(v)
+    valid = np.arange(seq)[None, :] < lens[:, None]
+    for got, exp, n in ((gq, eq, hn), (gk, ek, kvn), (gv, ev, kvn)):
+        pad = ~np.broadcast_to(valid[:, None, :, None], exp.shape)
+        assert np.array_equal(got[pad], exp[pad]), "padded positions must stay untouched"
+    assert np.array_equal(gv, ev), "v is a copy (+ bias in fp32 arithmetic): bit-exact"
+    if dtype == np.float32:
+        x = qkv.astype(np.float64)
+        if bias is not None:
+            x = x + bias.astype(np.float64).reshape(1, -1, hs)
+        half = hs // 2
+        rad = np.sqrt(x[..., :half] ** 2 + x[..., half:] ** 2)
+        rad = np.concatenate([rad, rad], axis=-1)  # [tokens, heads, hs]: the rotation radius of each pair
+        p = np.arange(tokens) + po
+        b, s = p // seq, p % seq
+        for got, exp, sl in ((gq, eq, slice(0, hn)), (gk, ek, slice(hn, hn + kvn))):
+            assert_f32_close(got[b, :, s, :], exp[b, :, s, :], "rotated heads", scale=rad[:, sl] + 1e-30)
+    else:
+        assert_f16_close(gq, eq, "q")
+        assert_f16_close(gk, ek, "k")
+    return lens
+
+
+def test_qkv_rope_config_fp16_b8_s512(isp, oracle):
+    lens = _check_qkv(isp, oracle, np.float16, 8, 512, 32, 32, 128, 128)
+    assert lens.min() >= 256 and lens.max() <= 512
+
+
+def test_qkv_rope_config_fp32_b8_s512(isp, oracle):
+    _check_qkv(isp, oracle, np.float32, 8, 512, 32, 32, 128, 128, seed=1)
+
+
+def test_qkv_rope_known_answer(isp):
+    # reference test: QKV = 32, offsets 0, history 0, seq 32 => q,k = 32 (cos a -/+ sin a), v = 32
+    S, hn, hs = 32, 32, 128
+    qkv = torch.full((S, 3 * hn, hs), 32.0, device="cuda")
+    q, k, v = (torch.zeros((1, hn, S, hs), device="cuda") for _ in range(3))
+    z = torch.zeros(S, dtype=torch.int32, device="cuda")
+    isp.add_fused_qkv_bias_transpose_and_rope(q, k, v, qkv, None, z, z[:1], z[:1] + 7, 128, 10000.0)
+    s = np.arange(S, dtype=np.float64)[:, None]
+    a = s / 10000.0 ** (np.arange(64, dtype=np.float64)[None, :] / 64.0)
+    exp = np.concatenate([32 * (np.cos(a) - np.sin(a)), 32 * (np.cos(a) + np.sin(a))], axis=1)
+    for t in (q, k):
+        assert_f32_close(host(t), np.broadcast_to(exp[None, None], (1, hn, S, hs)), "known answer",
+                         scale=np.full((1, hn, S, hs), 32 * np.sqrt(2.0)))
+    assert torch.all(v == 32.0)
+
+
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+@pytest.mark.parametrize("batch,seq,hn,kvn,hs,rot", [
+    (3, 12, 4, 4, 128, 128),    # vector path, tiny
+    (2, 9, 8, 2, 128, 128),     # GQA
+    (2, 9, 5, 1, 128, 64),      # MQA, partial rotary, head counts that do not fill a wave pass
+    (3, 7, 4, 2, 64, 64),       # 64-wide heads
+    (2, 6, 3, 3, 16, 16),       # scalar kernel
+    (2, 6, 2, 1, 96, 32),       # scalar kernel, partial rotary
+    (1, 1, 1, 1, 2, 2),         # smallest possible
+])
+def test_qkv_rope_shapes(isp, oracle, dtype, batch, seq, hn, kvn, hs, rot):
+    say("qkv %s b=%d s=%d hn=%d kvn=%d hs=%d rot=%d" % (dtype.__name__, batch, seq, hn, kvn, hs, rot))
+    hist = np.arange(batch, dtype=np.int32) * 5
+    _check_qkv(isp, oracle, dtype, batch, seq, hn, kvn, hs, rot, seed=batch * 100 + hs, min_len=0, history=hist)
+    _check_qkv(isp, oracle, dtype, batch, seq, hn, kvn, hs, rot, with_bias=False, seed=3, min_len=1)
+
+
+def test_qkv_rope_large_positions_fp32(isp, oracle):
+    # history pushes timesteps to ~4000: the angle must still match the oracle's fp32 angle exactly
+    _check_qkv(isp, oracle, np.float32, 2, 64, 4, 4, 128, 128, seed=8, history=[4000, 2500])
+
+
+def test_qkv_rope_skips_tokens_that_fall_outside(isp):
+    hn, hs, seq, batch = 2, 128, 4, 1
+    qkv = torch.ones((3, 3 * hn, hs), dtype=torch.float16, device="cuda")
+    q, k, v = (torch.zeros((batch, hn, seq, hs), dtype=torch.float16, device="cuda") for _ in range(3))
+    po = torch.tensor([0, 100, -50], dtype=torch.int32, device="cuda")  # tokens 1 and 2 land outside
+    z = torch.zeros(1, dtype=torch.int32, device="cuda")
+    isp.add_fused_qkv_bias_transpose_and_rope(q, k, v, qkv, None, po, z, z, 128, 10000.0)
+    torch.cuda.synchronize()
+    assert torch.all(v[0, :, 0] == 1) and torch.all(v[0, :, 1:] == 0)
