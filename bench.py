@@ -44,28 +44,45 @@ def parse():
 # --------------------------------------------------------------------------- workloads
 
 class Workload:
-    """One kernel at one shape: R rotating buffer sets and a launch(i) closure."""
+    """One kernel at one shape: R rotating buffer sets and a launch(i) closure.
+
+    launch(i) calls the C ABI directly with argument tuples prepared once (raw device pointers and
+    ints), so the per-launch host cost is one ctypes call; the small kernels are launch-bound and
+    every microsecond of host overhead would otherwise be billed to them."""
     name = ""
     dtype = ""
     tokens = 0
     bytes_per_launch = 0
-    kernel_symbol = ""
+    kernel = ""
+    sets = 1
+    keep = None
 
-    def sets_for(self, set_bytes, rotate):
+    @staticmethod
+    def sets_for(set_bytes, rotate):
         if not rotate:
             return 1
         return max(2, int((1 << 30) // max(set_bytes, 1)) + 1)
 
+    def bind(self, fn, arg_sets):
+        n = len(arg_sets)
+        self.sets = n
 
-def make_workloads(torch, ops, rotate):
+        def launch(i):
+            rc = fn(*arg_sets[i % n])
+            if rc:
+                raise RuntimeError("%s: C ABI returned %d" % (self.name, rc))
+        self.launch = launch
+
+
+def make_workloads(torch, lib, stream_handle, rotate):
     dev = "cuda"
-    W = []
+    st = stream_handle
 
     def norm(name, tokens, hidden, tdtype, fused):
         w = Workload()
         es = 2 if tdtype == torch.float16 else 4
-        w.name, w.dtype, w.tokens = name, ("f16" if es == 2 else "f32"), tokens
-        w.kernel_symbol = "fused_norm_rows"
+        sfx = "f16" if es == 2 else "f32"
+        w.name, w.dtype, w.tokens = name, sfx, tokens
         if fused:
             w.bytes_per_launch = 4 * tokens * hidden * es + 2 * hidden * es
             set_bytes = 2 * tokens * hidden * es
@@ -77,14 +94,15 @@ def make_workloads(torch, ops, rotate):
         ress = [torch.randn((tokens, hidden), device=dev, dtype=torch.float32).to(tdtype) for _ in range(R)] if fused else None
         bias = (0.02 * torch.randn(hidden, device=dev)).to(tdtype) if fused else None
         gamma = (0.5 + torch.rand(hidden, device=dev)).to(tdtype)
-        w.sets = R
-
-        def launch(i):
-            j = i % R
-            if fused:
-                ops.fused_add_bias_residual_rmsnorm(ress[j], outs[j], bias, gamma, 1e-5)
-            else:
-                ops.rmsnorm(outs[j], gamma, 1e-5)
+        w.keep = (outs, ress, bias, gamma)
+        w.kernel = "isp::fused_norm_rows<%s, ...>" % ("__half" if es == 2 else "float")
+        if fused:
+            fn = getattr(lib, "isp_fused_add_bias_residual_rmsnorm_" + sfx)
+            w.bind(fn, [(ress[j].data_ptr(), outs[j].data_ptr(), bias.data_ptr(), gamma.data_ptr(), 1e-5, tokens,
+                         hidden, 0, st) for j in range(R)])
+        else:
+            fn = getattr(lib, "isp_rmsnorm_" + sfx)
+            w.bind(fn, [(outs[j].data_ptr(), gamma.data_ptr(), 1e-5, tokens, hidden, st) for j in range(R)])
 
         def reset():
             # the kernel works in place: refresh the values so repeated launches stay finite
@@ -94,7 +112,7 @@ def make_workloads(torch, ops, rotate):
                 for t in ress:
                     t.normal_()
 
-        w.launch, w.reset = launch, reset
+        w.reset = reset
         w.config = {"tokens": tokens, "hidden": hidden}
         return w
 
@@ -102,14 +120,15 @@ def make_workloads(torch, ops, rotate):
         w = Workload()
         tokens, hidden, vocab = 8192, 4096, 32000
         w.name, w.dtype, w.tokens = "embedding_f16_8192x4096_v32000", "f16", tokens
-        w.kernel_symbol = "gather_rows_vec"
+        w.kernel = "isp::gather_chunks_vec<true>"
         w.bytes_per_launch = 2 * tokens * hidden * 2 + tokens * 4
         table = (0.02 * torch.randn((vocab, hidden), device=dev)).to(torch.float16)
         R = w.sets_for(tokens * hidden * 2, rotate)
         ids = [torch.randint(0, vocab, (tokens,), device=dev, dtype=torch.int32) for _ in range(R)]
         outs = [torch.empty((tokens, hidden), device=dev, dtype=torch.float16) for _ in range(R)]
-        w.sets = R
-        w.launch = lambda i: ops.input_embedding(ids[i % R], outs[i % R], table)
+        w.keep = (table, ids, outs)
+        w.bind(lib.isp_embedding_f16, [(ids[j].data_ptr(), outs[j].data_ptr(), table.data_ptr(), tokens, hidden,
+                                        vocab, st) for j in range(R)])
         w.reset = lambda: None
         w.config = {"tokens": tokens, "hidden": hidden, "vocab": vocab}
         return w
@@ -121,12 +140,13 @@ def make_workloads(torch, ops, rotate):
         lens = torch.randint(256, 513, (batch,), generator=g, dtype=torch.int32)
         tokens = int(lens.sum())
         w.name, w.dtype, w.tokens = "qkv_bias_rope_transpose_f16_b8_s512", "f16", tokens
-        w.kernel_symbol = "qkv_rope_vec"
+        w.kernel = "isp::qkv_rope_wave<__half, 128, true>"
         w.bytes_per_launch = tokens * (2 * (hn + 2 * kvn) * hs * 2 + 4) + (hn + 2 * kvn) * hs * 2 + 2 * batch * 4
         lens_d = lens.to(dev)
         po = torch.zeros((batch, seq), device=dev, dtype=torch.int32)
         cum = torch.zeros((batch + 1,), device=dev, dtype=torch.int32)
-        ops.cal_padding_offset(po, cum, lens_d)
+        rc = lib.isp_cal_padding_offset(po.data_ptr(), cum.data_ptr(), lens_d.data_ptr(), batch, seq, st)
+        assert rc == 0
         hist = torch.zeros(batch, device=dev, dtype=torch.int32)
         bias = (0.02 * torch.randn((hn + 2 * kvn) * hs, device=dev)).to(torch.float16)
         set_bytes = tokens * (hn + 2 * kvn) * hs * 2 + 3 * batch * hn * seq * hs * 2
@@ -134,14 +154,12 @@ def make_workloads(torch, ops, rotate):
         ins = [torch.randn((tokens, hn + 2 * kvn, hs), device=dev).to(torch.float16) for _ in range(R)]
         outs = [[torch.zeros((batch, n, seq, hs), device=dev, dtype=torch.float16) for n in (hn, kvn, kvn)]
                 for _ in range(R)]
-        w.sets = R
-
-        def launch(i):
-            j = i % R
-            ops.add_fused_qkv_bias_transpose_and_rope(outs[j][0], outs[j][1], outs[j][2], ins[j], bias, po, hist,
-                                                      lens_d, 128, 10000.0)
-
-        w.launch, w.reset = launch, (lambda: None)
+        w.keep = (lens_d, po, cum, hist, bias, ins, outs)
+        w.bind(lib.isp_qkv_bias_rope_transpose_f16,
+               [(outs[j][0].data_ptr(), outs[j][1].data_ptr(), outs[j][2].data_ptr(), ins[j].data_ptr(),
+                 bias.data_ptr(), po.data_ptr(), hist.data_ptr(), lens_d.data_ptr(), batch, seq, tokens, hn, kvn, hs,
+                 128, 10000.0, 2048, 0, st) for j in range(R)])
+        w.reset = lambda: None
         w.config = {"batch": batch, "max_seq": seq, "valid_tokens": tokens, "heads": "32q/32kv", "head_dim": hs}
         return w
 
@@ -149,18 +167,33 @@ def make_workloads(torch, ops, rotate):
         w = Workload()
         inter = 11008
         w.name, w.dtype, w.tokens = "swiglu_f16_%s_%dx%d" % (tag, tokens, inter), "f16", tokens
-        w.kernel_symbol = "swiglu_vec"
+        w.kernel = "isp::swiglu_vec<__half, 1, true>"
         w.bytes_per_launch = tokens * 3 * inter * 2
         R = w.sets_for(w.bytes_per_launch, rotate)
         ins = [torch.randn((tokens, 2, inter), device=dev).to(torch.float16) for _ in range(R)]
         outs = [torch.empty((tokens, inter), device=dev, dtype=torch.float16) for _ in range(R)]
-        w.sets = R
-        w.launch = lambda i: ops.act(ins[i % R], outs[i % R])
+        w.keep = (ins, outs)
+        w.bind(lib.isp_swiglu_f16, [(ins[j].data_ptr(), outs[j].data_ptr(), tokens, inter, st) for j in range(R)])
         w.reset = lambda: None
         w.config = {"tokens": tokens, "inter": inter}
         return w
 
-    makers = [
+    def copy(nbytes):
+        # calibration: a plain copy with the same traffic as the headline workload
+        w = Workload()
+        w.name, w.dtype, w.tokens = "calibration_copy_%dMiB_traffic" % (2 * nbytes >> 20), "u8", 0
+        w.kernel = "isp::copy_vec<4>"
+        w.bytes_per_launch = 2 * nbytes
+        R = w.sets_for(2 * nbytes, rotate)
+        srcs = [torch.empty(nbytes, device=dev, dtype=torch.uint8).fill_(j & 255) for j in range(R)]
+        dsts = [torch.empty(nbytes, device=dev, dtype=torch.uint8) for _ in range(R)]
+        w.keep = (srcs, dsts)
+        w.bind(lib.isp_calibration_copy, [(dsts[j].data_ptr(), srcs[j].data_ptr(), nbytes, st) for j in range(R)])
+        w.reset = lambda: None
+        w.config = {"bytes_copied": nbytes}
+        return w
+
+    return [
         ("fused_add_bias_residual_rmsnorm_f16_2048x4096",
          lambda: norm("fused_add_bias_residual_rmsnorm_f16_2048x4096", 2048, 4096, torch.float16, True)),
         ("rmsnorm_f32_64x4096", lambda: norm("rmsnorm_f32_64x4096", 64, 4096, torch.float32, False)),
@@ -169,8 +202,9 @@ def make_workloads(torch, ops, rotate):
         ("qkv_bias_rope_transpose_f16_b8_s512", qkv),
         ("swiglu_f16_prefill_8192x11008", lambda: swiglu(8192, "prefill")),
         ("swiglu_f16_decode_256x11008", lambda: swiglu(256, "decode")),
+        ("calibration_copy_64MiB_traffic", lambda: copy(32 << 20)),
+        ("calibration_copy_512MiB_traffic", lambda: copy(256 << 20)),
     ]
-    return makers
 
 
 # --------------------------------------------------------------------------- timing
@@ -198,35 +232,17 @@ def time_workload(torch, w, steps, warmup, stream):
     return wall_ms, event_ms
 
 
-def per_launch_event_ms(torch, w, steps, stream):
-    """Average of per-launch (event, launch, event) brackets: excludes most of the gap between
-    consecutive launches; reported next to the region average."""
-    n = min(steps, 100)
-    with torch.cuda.stream(stream):
-        w.reset()
-        torch.cuda.synchronize()
-        evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n)]
-        for i, (a, b) in enumerate(evs):
-            a.record(stream)
-            w.launch(i)
-            b.record(stream)
-        stream.synchronize()
-    ts = sorted(a.elapsed_time(b) for a, b in evs)
-    return sum(ts) / len(ts), ts[len(ts) // 2]
-
-
 def measure(torch, w, steps, warmup, stream):
     wall_ms, event_ms = time_workload(torch, w, steps, warmup, stream)
-    pl_mean, pl_median = per_launch_event_ms(torch, w, steps, stream)
     gbs = w.bytes_per_launch / (event_ms * 1e-3) / 1e9
     return {
-        "workload": w.name, "dtype": w.dtype, "tokens": w.tokens, "buffer_sets": w.sets,
+        "workload": w.name, "kernel": w.kernel, "dtype": w.dtype, "tokens": w.tokens, "buffer_sets": w.sets,
         "algorithmic_bytes": w.bytes_per_launch,
         "ms_per_step_wall": wall_ms, "ms_per_launch_events": event_ms,
-        "ms_per_launch_bracketed_mean": pl_mean, "ms_per_launch_bracketed_median": pl_median,
         "GBps": gbs, "frac_of_hbm_peak": gbs / HBM_PEAK_GBS,
-        "GBps_bracketed_median": w.bytes_per_launch / (pl_median * 1e-3) / 1e9,
-        "tokens_per_s": w.tokens / (event_ms * 1e-3),
+        "tokens_per_s": (w.tokens / (event_ms * 1e-3)) if w.tokens else None,
+        "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": gbs / HBM_PEAK_GBS, "traffic": None},
     }
 
 
@@ -287,45 +303,43 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py: no GPU available; the kernels have no CPU path", file=sys.stderr)
         sys.exit(3)
-    from inferspore_amd import capi, ops
-    capi.check(capi.lib().isp_init(), "isp_init")
+    from inferspore_amd import capi
+    lib = capi.lib()
+    capi.check(lib.isp_init(), "isp_init")
     torch.manual_seed(0)
     stream = torch.cuda.Stream()
+    handle = stream.cuda_stream
 
-    results, warm = [], {}
-    for name, make in make_workloads(torch, ops, True):
-        if a.only and a.only != name:
-            continue
-        w = make()
-        results.append(measure(torch, w, a.steps, a.warmup, stream))
-        del w
-        torch.cuda.empty_cache()
-    if a.warm:
-        for name, make in make_workloads(torch, ops, False):
+    def run_all(rotate):
+        out = []
+        for name, make in make_workloads(torch, lib, handle, rotate):
             if a.only and a.only != name:
                 continue
-            w = make()
-            m = measure(torch, w, a.steps, a.warmup, stream)
-            warm[name] = {"GBps": m["GBps"], "ms_per_launch_events": m["ms_per_launch_events"]}
+            with torch.cuda.stream(stream):
+                w = make()
+            torch.cuda.synchronize()
+            out.append(measure(torch, w, a.steps, a.warmup, stream))
             del w
             torch.cuda.empty_cache()
+        return out
+
+    results = run_all(True)
     head = results[0]
     line = {
         "metric": "HBM GB/s & % of peak per fused kernel at LLaMA-2-7B shapes; tokens/sec",
         "value": head["GBps"], "unit": "GB/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
         "ms_per_step": head["ms_per_step_wall"], "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "f16 storage / f32 arithmetic", "data": "synthetic",
+        "vs_baseline": None, "dtype": "f16 storage, f32 arithmetic", "data": "synthetic",
         "config": {"workload": head["workload"], "tokens_per_s": head["tokens_per_s"],
-                   "cache": "cold (rotating %d buffer sets > 1 GiB)" % head["buffer_sets"]},
-        "roofline": {"bound": "hbm", "achieved": head["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": head["GBps"] / HBM_PEAK_GBS, "traffic": None,
-                     "kernel": "fused_norm_rows<__half, 2, 4>",
-                     "algorithmic_bytes_per_launch": head["algorithmic_bytes"],
-                     "avg_launch_ms": head["ms_per_launch_events"]},
+                   "cache": "cold: launches rotate over %d buffer sets (> 1 GiB)" % head["buffer_sets"]},
+        "roofline": dict(head["roofline"], kernel=head["kernel"],
+                         algorithmic_bytes_per_launch=head["algorithmic_bytes"],
+                         avg_launch_ms=head["ms_per_launch_events"]),
         "kernels": results,
     }
-    if warm:
-        line["warm_cache"] = warm
+    if a.warm:
+        line["warm_cache"] = {r["workload"]: {"GBps": r["GBps"], "ms_per_launch_events": r["ms_per_launch_events"]}
+                              for r in run_all(False)}
     if not a.no_cpu:
         line["cpu_baseline"] = cpu_baseline(a.cpu_seconds)
     print(json.dumps(line))

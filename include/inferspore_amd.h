@@ -24,6 +24,7 @@
 #ifndef INFERSPORE_AMD_H
 #define INFERSPORE_AMD_H
 
+#include <stddef.h>
 #include <stdint.h>
 
 #ifdef __cplusplus
@@ -139,6 +140,30 @@ int isp_qkv_bias_rope_transpose_f16(void* q, void* k, void* v, const void* qkv, 
  */
 int isp_swiglu_f32(const void* in, void* out, int tokens, int inter, isp_stream_t stream);
 int isp_swiglu_f16(const void* in, void* out, int tokens, int inter, isp_stream_t stream);
+
+/*
+ * Measurement aids (no reference counterpart).
+ * isp_calibration_copy: a plain copy kernel of known traffic (`bytes` read + `bytes` written;
+ *   16-byte aligned, multiple of 16) used to calibrate profiler byte counters and to measure the
+ *   copy bandwidth the machine actually reaches.
+ * isp_tuning_set: overrides a launch heuristic process-wide (0 restores the automatic choice) and
+ *   returns the previous value, or ISP_ERR_BAD_SHAPE for an unknown knob.  For benchmark sweeps;
+ *   results never depend on the knobs, only speed does.
+ */
+int isp_calibration_copy(void* dst, const void* src, size_t bytes, isp_stream_t stream);
+
+typedef enum isp_tuning_knob {
+    ISP_TUNE_NORM_WAVES_PER_ROW = 0, /* 1, 2, 4, 8 or 16 waves cooperate on one token row */
+    ISP_TUNE_NORM_STORE = 1,         /* output stores: 1 = plain, 2 = non-temporal (default) */
+    ISP_TUNE_SWIGLU_UNROLL = 2,      /* 1 (default), 2 or 4 vector pairs in flight per lane */
+    ISP_TUNE_SWIGLU_STORE = 3,       /* 1 = plain, 2 = non-temporal (default) */
+    ISP_TUNE_EMBED_VARIANT = 4,      /* 1 = a wave per row, 2 = a workgroup per row,
+                                        3 = a workgroup per 4 KiB chunk of a row (default) */
+    ISP_TUNE_EMBED_STORE = 5,        /* 1 = plain, 2 = non-temporal (default) */
+    ISP_TUNE_QKV_STORE = 6,          /* 1 = plain, 2 = non-temporal (default) */
+    ISP_TUNE_COUNT = 7
+} isp_tuning_knob;
+int isp_tuning_set(int knob, int value);
 
 #ifdef __cplusplus
 }

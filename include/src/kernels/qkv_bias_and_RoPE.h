@@ -1,0 +1,17 @@
+// launchAddFusedQKVBiasTransposeAndRoPE -- same declaration as the reference's
+// src/kernels/qkv_bias_and_RoPE.h:10-20.  Shapes are taken from the tensors as the reference's
+// launcher does (src/kernels/qkv_bias_and_RoPE.cu:298-304):
+//   QKV [token_num, head_num + 2 kv_head_num, head_size];  q_buf [batch, head_num, seq_len, head_size];
+//   k_buf, v_buf [batch, kv_head_num, seq_len, head_size];  bias = qkv.bias (may be null).
+#pragma once
+#include "src/models/llama/llama_params.h"
+#include "src/utils/tensor.h"
+#include "src/utils/vectorize_utils.h"
+#include "src/weights/base_weights.h"
+template <typename T>
+void launchAddFusedQKVBiasTransposeAndRoPE(TensorWrapper<T>* q_buf, TensorWrapper<T>* k_buf,
+                                           TensorWrapper<T>* v_buf, TensorWrapper<T>* QKV,
+                                           BaseWeight<T>& qkv, TensorWrapper<int>* padding_offset,
+                                           TensorWrapper<int>* history_length,
+                                           TensorWrapper<int>* input_length,
+                                           LLaMAAttentionStaticParams& params);

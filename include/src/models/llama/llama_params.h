@@ -1,0 +1,11 @@
+// Static attention parameters.  The reference includes "src/models/llama/llama_params.h" from
+// src/kernels/qkv_bias_and_RoPE.h:5 but ships no such file; the members are the ones its code
+// assigns and reads (src/kernels/qkv_bias_and_RoPE.cu:322-325,
+// tests/unittests/test_bias_and_RoPE.cu:163-167, src/utils/model_utils.h:25-29).
+#pragma once
+struct LLaMAAttentionStaticParams {
+    int rotary_embedding_dim = 128;
+    float rotary_embedding_base = 10000.0f;
+    int max_position_embeddings = 2048;
+    bool use_dynamic_ntk = false;  // placeholder in the reference as well
+};

@@ -12,6 +12,8 @@ ERR_UNSUPPORTED = -3
 ERR_LAUNCH = -4
 ERR_DEVICE = -5
 NORM_RESIDUAL_EXCLUDES_BIAS = 1
+(TUNE_NORM_WAVES_PER_ROW, TUNE_NORM_STORE, TUNE_SWIGLU_UNROLL, TUNE_SWIGLU_STORE, TUNE_EMBED_VARIANT,
+ TUNE_EMBED_STORE, TUNE_QKV_STORE) = range(7)
 
 _vp, _i, _f, _u = C.c_void_p, C.c_int, C.c_float, C.c_uint
 
@@ -32,7 +34,8 @@ SIGNATURES = {
     "isp_qkv_bias_rope_transpose_f16": (_i, [_vp] * 8 + [_i] * 7 + [_f, _i, _i, _vp]),
     "isp_swiglu_f32": (_i, [_vp, _vp, _i, _i, _vp]),
     "isp_swiglu_f16": (_i, [_vp, _vp, _i, _i, _vp]),
-    "isp_tuning_norm_waves_per_row": (_i, [_i]),
+    "isp_tuning_set": (_i, [_i, _i]),
+    "isp_calibration_copy": (_i, [_vp, _vp, C.c_size_t, _vp]),
 }
 
 _lib = None

@@ -13,9 +13,20 @@ int note_launch(hipError_t e) {
     return ISP_ERR_LAUNCH;
 }
 
+static int g_tuning[ISP_TUNE_COUNT] = {0};
+
+int tuning(int knob) { return (knob >= 0 && knob < ISP_TUNE_COUNT) ? g_tuning[knob] : 0; }
+
 }  // namespace isp
 
 extern "C" {
+
+int isp_tuning_set(int knob, int value) {
+    if (knob < 0 || knob >= ISP_TUNE_COUNT) return ISP_ERR_BAD_SHAPE;
+    const int old = isp::g_tuning[knob];
+    isp::g_tuning[knob] = value;
+    return old;
+}
 
 const char* isp_version(void) { return "inferspore_amd 0.1 (gfx950)"; }
 

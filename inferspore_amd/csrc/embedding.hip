@@ -2,32 +2,36 @@
 //
 // Semantics: src/kernels/input_embedding.cu:14-21.  It is a raw row copy, so one kernel serves every
 // element type (the row is handled as bytes) and the result is bit-exact by construction.
-// Design: one wave per token row; the token id is read once per row into a scalar register (the
-// reference re-reads ids[] and does a div/mod for every 2-byte element); the row moves as 16-byte
-// vectors with eight loads in flight per lane; four rows per workgroup.
+// Design: the token id is read once per workgroup into a scalar register (the reference re-reads
+// ids[] and does a div/mod for every 2-byte element) and the row moves as 16-byte vectors, one
+// vector per lane, one 4 KiB chunk of a row per workgroup -- the access order that streams best on
+// this memory system; wave-per-row and workgroup-per-row variants remain selectable for sweeps.
 #include "isp_common.h"
 
 namespace isp {
 
-template <int UNROLL>
+// ROW_THREADS lanes (a wave, or the whole workgroup) share one row; each lane moves UNROLL vectors
+// per trip, strided by ROW_THREADS.
+template <int ROW_THREADS, int UNROLL, bool NT>
 __global__ __launch_bounds__(kBlock) void gather_rows_vec(const int32_t* __restrict__ ids,
                                                           char* __restrict__ out,
                                                           const char* __restrict__ table, int tokens,
                                                           unsigned row_vec, int vocab) {
-    const int wave = threadIdx.x / kWave;
-    const int lane = threadIdx.x % kWave;
-    const int row = blockIdx.x * (kBlock / kWave) + wave;
-    if (row >= tokens) return;  // whole wave leaves together; no barrier follows
+    constexpr int ROWS = kBlock / ROW_THREADS;
+    const int slot = threadIdx.x / ROW_THREADS;
+    const int lane = threadIdx.x % ROW_THREADS;
+    const int row = blockIdx.x * ROWS + slot;
+    if (row >= tokens) return;  // whole waves leave together; no barrier follows
     const int id = __builtin_amdgcn_readfirstlane(ids[row]);
     const bool in_range = vocab <= 0 || (id >= 0 && id < vocab);
     const size_t row_bytes = (size_t)row_vec * 16u;
     const char* src = table + (size_t)(in_range ? id : 0) * row_bytes;
     char* dst = out + (size_t)row * row_bytes;
-    for (unsigned v0 = lane; v0 < row_vec; v0 += kWave * UNROLL) {
+    for (unsigned v0 = lane; v0 < row_vec; v0 += ROW_THREADS * UNROLL) {
         vec16 buf[UNROLL];
 #pragma unroll
         for (int k = 0; k < UNROLL; k++) {
-            const unsigned v = v0 + k * kWave;
+            const unsigned v = v0 + k * ROW_THREADS;
             if (v < row_vec) {
                 if (in_range) {
                     buf[k] = load16_stream(src + (size_t)v * 16u);
@@ -38,10 +42,29 @@ __global__ __launch_bounds__(kBlock) void gather_rows_vec(const int32_t* __restr
         }
 #pragma unroll
         for (int k = 0; k < UNROLL; k++) {
-            const unsigned v = v0 + k * kWave;
-            if (v < row_vec) store16(dst + (size_t)v * 16u, buf[k]);
+            const unsigned v = v0 + k * ROW_THREADS;
+            if (v < row_vec) store16_sel<NT>(dst + (size_t)v * 16u, buf[k]);
         }
     }
+}
+
+// One 16-byte vector per lane: a workgroup moves one 4 KiB chunk of one row.
+template <bool NT>
+__global__ __launch_bounds__(kBlock) void gather_chunks_vec(const int32_t* __restrict__ ids,
+                                                            char* __restrict__ out,
+                                                            const char* __restrict__ table,
+                                                            unsigned chunks_per_row,
+                                                            unsigned row_vec, int vocab) {
+    const unsigned row = blockIdx.x / chunks_per_row;
+    const unsigned v = (blockIdx.x % chunks_per_row) * kBlock + threadIdx.x;
+    if (v >= row_vec) return;
+    const int id = __builtin_amdgcn_readfirstlane(ids[row]);
+    const bool in_range = vocab <= 0 || (id >= 0 && id < vocab);
+    const size_t row_bytes = (size_t)row_vec * 16u;
+    vec16 buf;
+    if (in_range) buf = load16_stream(table + (size_t)id * row_bytes + (size_t)v * 16u);
+    else buf.w[0] = buf.w[1] = buf.w[2] = buf.w[3] = 0u;
+    store16_sel<NT>(out + (size_t)row * row_bytes + (size_t)v * 16u, buf);
 }
 
 // Rows that are not a whole number of aligned 16-byte vectors: one workgroup per row, byte copies.
@@ -66,11 +89,25 @@ static int embedding(const int32_t* ids, void* out, const void* table, int token
     const size_t row_bytes = (size_t)hidden * (size_t)elem_size;
     hipError_t e;
     if (row_bytes % 16 == 0 && aligned16(out) && aligned16(table)) {
-        constexpr int ROWS = kBlock / kWave;
-        dim3 grid((unsigned)((tokens + ROWS - 1) / ROWS));
-        hipLaunchKernelGGL((gather_rows_vec<8>), grid, dim3(kBlock), 0, s, ids,
-                           static_cast<char*>(out), static_cast<const char*>(table), tokens,
-                           (unsigned)(row_bytes / 16), vocab);
+        const bool nt = tuning(ISP_TUNE_EMBED_STORE) != 1;
+        const unsigned row_vec = (unsigned)(row_bytes / 16);
+        char* o = static_cast<char*>(out);
+        const char* t = static_cast<const char*>(table);
+        const int variant = tuning(ISP_TUNE_EMBED_VARIANT);
+        if (variant == 1) {  // one wave per row
+            dim3 grid((unsigned)((tokens + 3) / 4)), block(kBlock);
+            if (nt) hipLaunchKernelGGL((gather_rows_vec<kWave, 4, true>), grid, block, 0, s, ids, o, t, tokens, row_vec, vocab);
+            else hipLaunchKernelGGL((gather_rows_vec<kWave, 4, false>), grid, block, 0, s, ids, o, t, tokens, row_vec, vocab);
+        } else if (variant == 2 || (size_t)tokens * ((row_vec + kBlock - 1) / kBlock) > 0x7fffffffull) {
+            dim3 grid((unsigned)tokens), block(kBlock);  // one workgroup per row
+            if (nt) hipLaunchKernelGGL((gather_rows_vec<kBlock, 2, true>), grid, block, 0, s, ids, o, t, tokens, row_vec, vocab);
+            else hipLaunchKernelGGL((gather_rows_vec<kBlock, 2, false>), grid, block, 0, s, ids, o, t, tokens, row_vec, vocab);
+        } else {  // one 4 KiB chunk of a row per workgroup, one vector per lane
+            const unsigned chunks = (row_vec + kBlock - 1) / kBlock;
+            dim3 grid((unsigned)tokens * chunks), block(kBlock);
+            if (nt) hipLaunchKernelGGL((gather_chunks_vec<true>), grid, block, 0, s, ids, o, t, chunks, row_vec, vocab);
+            else hipLaunchKernelGGL((gather_chunks_vec<false>), grid, block, 0, s, ids, o, t, chunks, row_vec, vocab);
+        }
         e = hipGetLastError();
     } else {
         hipLaunchKernelGGL(gather_rows_bytes, dim3((unsigned)tokens), dim3(kBlock), 0, s, ids,

@@ -17,6 +17,9 @@ constexpr int kBlock = 256;   // threads per workgroup used by every kernel here
 // Records a failed launch for isp_last_hip_error(); returns the status to hand back.
 int note_launch(hipError_t e);
 
+// Current value of a tuning knob (isp_tuning_set); 0 means "automatic" for every knob.
+int tuning(int knob);
+
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 #define ISP_REQUIRE_PTR(p)                   \
@@ -51,6 +54,11 @@ __device__ __forceinline__ void store16_stream(void* p, const vec16& v) {
     typedef uint32_t u4 __attribute__((ext_vector_type(4)));
     u4 t = {v.w[0], v.w[1], v.w[2], v.w[3]};
     __builtin_nontemporal_store(t, reinterpret_cast<u4*>(p));
+}
+
+template <bool NT>
+__device__ __forceinline__ void store16_sel(void* p, const vec16& v) {
+    if (NT) store16_stream(p, v); else store16(p, v);
 }
 
 // Element traits: how many elements a 16-byte vector holds and how to move between storage and fp32.

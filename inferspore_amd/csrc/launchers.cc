@@ -1,0 +1,133 @@
+// The reference's C++ launch* entry points, as thin shims over the C ABI (inferspore_amd.h).
+// Each shim unpacks shapes and pointers from the TensorWrapper / weight structs the way the
+// reference's launcher does (cited per function), keeps the reference's own argument checks, and
+// launches on the null stream like the reference.  A non-zero status from the C ABI becomes the
+// same std::runtime_error the reference's LLM_CHECK raises.
+#include "inferspore_amd.h"
+#include "src/kernels/act_kernel.h"
+#include "src/kernels/cal_paddingoffset.h"
+#include "src/kernels/fused_addresidual_norm.h"
+#include "src/kernels/input_embedding.h"
+#include "src/kernels/qkv_bias_and_RoPE.h"
+#include "src/kernels/rmsnorm.h"
+
+namespace {
+
+template <typename T>
+struct Abi;
+template <>
+struct Abi<float> {
+    static constexpr auto embedding = isp_embedding_f32;
+    static constexpr auto rmsnorm = isp_rmsnorm_f32;
+    static constexpr auto fused_norm = isp_fused_add_bias_residual_rmsnorm_f32;
+    static constexpr auto qkv = isp_qkv_bias_rope_transpose_f32;
+    static constexpr auto swiglu = isp_swiglu_f32;
+};
+template <>
+struct Abi<half> {
+    static constexpr auto embedding = isp_embedding_f16;
+    static constexpr auto rmsnorm = isp_rmsnorm_f16;
+    static constexpr auto fused_norm = isp_fused_add_bias_residual_rmsnorm_f16;
+    static constexpr auto qkv = isp_qkv_bias_rope_transpose_f16;
+    static constexpr auto swiglu = isp_swiglu_f16;
+};
+
+inline void expect_ok(int status, const char* what) {
+    LLM_CHECK_WITH_INFO(status == ISP_OK, std::string(what) + ": " + isp_strerror(status));
+}
+
+}  // namespace
+
+// reference: src/kernels/input_embedding.cu:25-45 (token count and hidden size from output->shape,
+// the shape check at :35)
+template <typename T>
+void launchInputEmbedding(TensorWrapper<int>* input_ids, TensorWrapper<T>* output,
+                          EmbeddingWeight<T>* embed_table) {
+    const int tokens = output->shape[0];
+    const int hidden = output->shape[1];
+    LLM_CHECK_WITH_INFO(tokens == input_ids->shape[0],
+                        "input ids 1st shape should equal to 1st shape of output");
+    const int vocab = embed_table->shape.size() == 2 ? embed_table->shape[0] : 0;
+    expect_ok(Abi<T>::embedding(input_ids->data, output->data, embed_table->data, tokens, hidden,
+                                vocab, nullptr),
+              "launchInputEmbedding");
+}
+
+// reference: src/kernels/cal_paddingoffset.cu:49-60
+void launchCalPaddingoffset(TensorWrapper<int>* padding_offset, TensorWrapper<int>* cum_seqlens,
+                            TensorWrapper<int>* input_lengths) {
+    const int batch = padding_offset->shape[0];
+    const int max_q_len = padding_offset->shape[1];
+    LLM_CHECK_WITH_INFO(batch == input_lengths->shape[0],
+                        "input lenghts numbers should equal to padding offset bs dim!");
+    LLM_CHECK_WITH_INFO(batch == cum_seqlens->shape[0] - 1,
+                        "cum seqlen numbers should equal to padding offset bs dim + 1!");
+    expect_ok(isp_cal_padding_offset(padding_offset->data, cum_seqlens->data, input_lengths->data,
+                                     batch, max_q_len, nullptr),
+              "launchCalPaddingoffset");
+}
+
+// reference: src/kernels/fused_addresidual_norm.cu:143-170 (tokens, hidden from decoder_out->shape;
+// bias = norm.bias; gamma = scale)
+template <typename T>
+void launchFusedAddBiasResidualRMSNorm(TensorWrapper<T>* residual, TensorWrapper<T>* decoder_out,
+                                       BaseWeight<T>& norm, T* scale, float eps) {
+    const int tokens = decoder_out->shape[0];
+    const int hidden = decoder_out->shape[1];
+    expect_ok(Abi<T>::fused_norm(residual->data, decoder_out->data, norm.bias, scale, eps, tokens,
+                                 hidden, 0u, nullptr),
+              "launchFusedAddBiasResidualRMSNorm");
+}
+
+template <typename T>
+void launchRMSNorm(TensorWrapper<T>* decoder_out, LayerNormWeight<T>& norm, float eps) {
+    expect_ok(Abi<T>::rmsnorm(decoder_out->data, norm.gamma, eps, decoder_out->shape[0],
+                              decoder_out->shape[1], nullptr),
+              "launchRMSNorm");
+}
+
+// reference: src/kernels/qkv_bias_and_RoPE.cu:286-330 (shape derivation :298-304)
+template <typename T>
+void launchAddFusedQKVBiasTransposeAndRoPE(TensorWrapper<T>* q_buf, TensorWrapper<T>* k_buf,
+                                           TensorWrapper<T>* v_buf, TensorWrapper<T>* QKV,
+                                           BaseWeight<T>& qkv, TensorWrapper<int>* padding_offset,
+                                           TensorWrapper<int>* history_length,
+                                           TensorWrapper<int>* input_length,
+                                           LLaMAAttentionStaticParams& params) {
+    const int token_num = QKV->shape[0];
+    const int qkv_head_num = QKV->shape[1];
+    const int head_size = QKV->shape[2];
+    const int batch_size = q_buf->shape[0];
+    const int head_num = q_buf->shape[1];
+    const int seq_len = q_buf->shape[2];
+    const int kv_head_num = (qkv_head_num - head_num) / 2;
+    expect_ok(Abi<T>::qkv(q_buf->data, k_buf->data, v_buf->data, QKV->data, qkv.bias,
+                          padding_offset->data, history_length->data, input_length->data,
+                          batch_size, seq_len, token_num, head_num, kv_head_num, head_size,
+                          params.rotary_embedding_dim, params.rotary_embedding_base,
+                          params.max_position_embeddings, params.use_dynamic_ntk ? 1 : 0, nullptr),
+              "launchAddFusedQKVBiasTransposeAndRoPE");
+}
+
+// reference: src/kernels/act_kernel.cu:57-71 (the shape[1] == 2 check at :61)
+template <typename T>
+void launchAct(TensorWrapper<T>* input, TensorWrapper<T>* out) {
+    const int tokens = input->shape[0];
+    LLM_CHECK(input->shape[1] == 2);
+    const int inter = input->shape[2];
+    expect_ok(Abi<T>::swiglu(input->data, out->data, tokens, inter, nullptr), "launchAct");
+}
+
+// explicit instantiations for float and half, as in the reference
+#define ISP_INSTANTIATE(T)                                                                          \
+    template void launchInputEmbedding(TensorWrapper<int>*, TensorWrapper<T>*, EmbeddingWeight<T>*); \
+    template void launchFusedAddBiasResidualRMSNorm(TensorWrapper<T>*, TensorWrapper<T>*,           \
+                                                    BaseWeight<T>&, T*, float);                     \
+    template void launchRMSNorm(TensorWrapper<T>*, LayerNormWeight<T>&, float);                     \
+    template void launchAddFusedQKVBiasTransposeAndRoPE(                                            \
+        TensorWrapper<T>*, TensorWrapper<T>*, TensorWrapper<T>*, TensorWrapper<T>*, BaseWeight<T>&, \
+        TensorWrapper<int>*, TensorWrapper<int>*, TensorWrapper<int>*, LLaMAAttentionStaticParams&); \
+    template void launchAct(TensorWrapper<T>*, TensorWrapper<T>*);
+ISP_INSTANTIATE(float)
+ISP_INSTANTIATE(half)
+#undef ISP_INSTANTIATE

@@ -11,18 +11,23 @@
 
 namespace isp {
 
-// One row is handled by WPR waves (ROW_THREADS = 64 * WPR lanes); a 256-thread workgroup therefore
-// carries 4 / WPR rows.  Each lane owns NV 16-byte vectors of the row, strided by ROW_THREADS so
-// that every load instruction of a wave covers 1 KiB of contiguous memory.
-template <typename T, int NV, int WPR>
-__global__ __launch_bounds__(kBlock) void fused_norm_rows(T* __restrict__ residual,
-                                                          T* __restrict__ out,
-                                                          const T* __restrict__ bias,
-                                                          const T* __restrict__ gamma, float eps,
-                                                          int tokens, int hidden, unsigned flags) {
+// One row is handled by WPR waves (ROW_THREADS = 64 * WPR lanes); a workgroup has at least 256
+// threads and therefore carries 4 / WPR rows when WPR < 4.  Each lane owns NV 16-byte vectors of
+// the row, strided by ROW_THREADS so that every load instruction of a wave covers 1 KiB of
+// contiguous memory.  NT selects non-temporal stores for the two outputs.
+constexpr int norm_block(int wpr) { return kWave * wpr > kBlock ? kWave * wpr : kBlock; }
+
+template <typename T, int NV, int WPR, bool NT>
+__global__ __launch_bounds__(norm_block(WPR)) void fused_norm_rows(T* __restrict__ residual,
+                                                                   T* __restrict__ out,
+                                                                   const T* __restrict__ bias,
+                                                                   const T* __restrict__ gamma,
+                                                                   float eps, int tokens, int hidden,
+                                                                   unsigned flags) {
     constexpr int VEC = Elem<T>::kVec;
     constexpr int ROW_THREADS = kWave * WPR;
-    constexpr int ROWS = kBlock / ROW_THREADS;
+    constexpr int BLOCK = norm_block(WPR);
+    constexpr int ROWS = BLOCK / ROW_THREADS;
 
     const int slot = threadIdx.x / ROW_THREADS;
     const int lane = threadIdx.x % ROW_THREADS;
@@ -58,7 +63,7 @@ __global__ __launch_bounds__(kBlock) void fused_norm_rows(T* __restrict__ residu
 #pragma unroll
                 for (int e = 0; e < VEC; e++) x[j][e] += r[e];
                 if (flags & ISP_NORM_RESIDUAL_EXCLUDES_BIAS)
-                    store16(rsd_row + (size_t)vi * VEC, Elem<T>::pack(x[j]));
+                    store16_sel<NT>(rsd_row + (size_t)vi * VEC, Elem<T>::pack(x[j]));
             }
             if (bias) {
                 float b[VEC];
@@ -67,7 +72,7 @@ __global__ __launch_bounds__(kBlock) void fused_norm_rows(T* __restrict__ residu
                 for (int e = 0; e < VEC; e++) x[j][e] += b[e];
             }
             if (rsd_row && !(flags & ISP_NORM_RESIDUAL_EXCLUDES_BIAS))
-                store16(rsd_row + (size_t)vi * VEC, Elem<T>::pack(x[j]));
+                store16_sel<NT>(rsd_row + (size_t)vi * VEC, Elem<T>::pack(x[j]));
 #pragma unroll
             for (int e = 0; e < VEC; e++) acc += x[j][e] * x[j][e];
         }
@@ -75,7 +80,7 @@ __global__ __launch_bounds__(kBlock) void fused_norm_rows(T* __restrict__ residu
 
     float total = wave_sum(acc);
     if (WPR > 1) {
-        __shared__ float partial[kBlock / kWave];
+        __shared__ float partial[BLOCK / kWave];
         const int wave = threadIdx.x / kWave;
         if ((threadIdx.x % kWave) == 0) partial[wave] = total;
         __syncthreads();
@@ -94,7 +99,7 @@ __global__ __launch_bounds__(kBlock) void fused_norm_rows(T* __restrict__ residu
             float y[VEC];
 #pragma unroll
             for (int e = 0; e < VEC; e++) y[e] = g[e] * x[j][e] * inv;
-            store16(out_row + (size_t)vi * VEC, Elem<T>::pack(y));
+            store16_sel<NT>(out_row + (size_t)vi * VEC, Elem<T>::pack(y));
         }
     }
 }
@@ -134,28 +139,41 @@ __global__ __launch_bounds__(kBlock) void fused_norm_generic(T* residual, T* out
     }
 }
 
-template <typename T, int NV, int WPR>
+template <typename T, int NV, int WPR, bool NT>
 static hipError_t launch_rows(T* residual, T* out, const T* bias, const T* gamma, float eps,
                               int tokens, int hidden, unsigned flags, hipStream_t s) {
-    constexpr int ROWS = kBlock / (kWave * WPR);
+    constexpr int BLOCK = norm_block(WPR);
+    constexpr int ROWS = BLOCK / (kWave * WPR);
     dim3 grid((unsigned)((tokens + ROWS - 1) / ROWS));
-    hipLaunchKernelGGL((fused_norm_rows<T, NV, WPR>), grid, dim3(kBlock), 0, s, residual, out, bias,
-                       gamma, eps, tokens, hidden, flags);
+    hipLaunchKernelGGL((fused_norm_rows<T, NV, WPR, NT>), grid, dim3(BLOCK), 0, s, residual, out,
+                       bias, gamma, eps, tokens, hidden, flags);
     return hipGetLastError();
 }
 
-template <typename T, int WPR>
+template <typename T, int WPR, bool NT>
 static hipError_t launch_rows_nv(int nv, T* residual, T* out, const T* bias, const T* gamma,
                                  float eps, int tokens, int hidden, unsigned flags, hipStream_t s) {
-    if (nv <= 1) return launch_rows<T, 1, WPR>(residual, out, bias, gamma, eps, tokens, hidden, flags, s);
-    if (nv <= 2) return launch_rows<T, 2, WPR>(residual, out, bias, gamma, eps, tokens, hidden, flags, s);
-    if (nv <= 4) return launch_rows<T, 4, WPR>(residual, out, bias, gamma, eps, tokens, hidden, flags, s);
-    return launch_rows<T, 8, WPR>(residual, out, bias, gamma, eps, tokens, hidden, flags, s);
+    if (nv <= 1) return launch_rows<T, 1, WPR, NT>(residual, out, bias, gamma, eps, tokens, hidden, flags, s);
+    if (nv <= 2) return launch_rows<T, 2, WPR, NT>(residual, out, bias, gamma, eps, tokens, hidden, flags, s);
+    if (nv <= 4) return launch_rows<T, 4, WPR, NT>(residual, out, bias, gamma, eps, tokens, hidden, flags, s);
+    return launch_rows<T, 8, WPR, NT>(residual, out, bias, gamma, eps, tokens, hidden, flags, s);
 }
 
-// Waves per row: rows per workgroup trade against loads in flight per lane.  tuning_wpr() lets the
-// benchmark sweep the choice (0 = automatic).
-static int g_norm_wpr = 0;
+template <typename T, bool NT>
+static hipError_t launch_rows_wpr(int wpr, int nv, T* residual, T* out, const T* bias,
+                                  const T* gamma, float eps, int tokens, int hidden, unsigned flags,
+                                  hipStream_t s) {
+    switch (wpr) {
+        case 1: return launch_rows_nv<T, 1, NT>(nv, residual, out, bias, gamma, eps, tokens, hidden, flags, s);
+        case 2: return launch_rows_nv<T, 2, NT>(nv, residual, out, bias, gamma, eps, tokens, hidden, flags, s);
+        case 4: return launch_rows_nv<T, 4, NT>(nv, residual, out, bias, gamma, eps, tokens, hidden, flags, s);
+        case 8: return launch_rows_nv<T, 8, NT>(nv, residual, out, bias, gamma, eps, tokens, hidden, flags, s);
+        default: return launch_rows_nv<T, 16, NT>(nv, residual, out, bias, gamma, eps, tokens, hidden, flags, s);
+    }
+}
+
+constexpr int kMaxWpr = 16;  // 1024 threads
+constexpr int kMaxNv = 8;
 
 template <typename T>
 static int fused_norm(void* residual_, void* out_, const void* bias_, const void* gamma_, float eps,
@@ -169,11 +187,10 @@ static int fused_norm(void* residual_, void* out_, const void* bias_, const void
     const T* bias = static_cast<const T*>(bias_);
     const T* gamma = static_cast<const T*>(gamma_);
     constexpr int VEC = Elem<T>::kVec;
-    constexpr int MAX_NV = 8;
 
     const bool vec_ok = (hidden % VEC == 0) && aligned16(out) && aligned16(gamma) &&
                         (!residual || aligned16(residual)) && (!bias || aligned16(bias)) &&
-                        (hidden / VEC) <= MAX_NV * kBlock;
+                        (hidden / VEC) <= kMaxNv * kWave * kMaxWpr;
     hipError_t e;
     if (!vec_ok) {
         hipLaunchKernelGGL((fused_norm_generic<T>), dim3((unsigned)tokens), dim3(kBlock), 0, s,
@@ -181,20 +198,22 @@ static int fused_norm(void* residual_, void* out_, const void* bias_, const void
         e = hipGetLastError();
     } else {
         const int nvec = hidden / VEC;
-        int wpr = g_norm_wpr;
-        if (wpr != 1 && wpr != 2 && wpr != 4) {
-            // automatic: the fewest waves per row that keep at most 4 vectors per lane in flight
+        auto vectors_per_lane = [nvec](int w) { return (nvec + kWave * w - 1) / (kWave * w); };
+        int wpr = tuning(ISP_TUNE_NORM_WAVES_PER_ROW);
+        if (wpr != 1 && wpr != 2 && wpr != 4 && wpr != 8 && wpr != 16) {
+            // automatic: the fewest waves per row that leave at most 2 vectors per lane; when there
+            // are too few rows to occupy the machine (4 waves on each of 1024 SIMDs), split rows
+            // further, down to one vector per lane
             wpr = 1;
-            while (wpr < 4 && (nvec + kWave * wpr - 1) / (kWave * wpr) > 4) wpr *= 2;
+            while (wpr < kMaxWpr && vectors_per_lane(wpr) > 2) wpr *= 2;
+            while (wpr < kMaxWpr && vectors_per_lane(wpr) > 1 && (long long)tokens * wpr < 4096) wpr *= 2;
         }
-        while (wpr < 4 && (nvec + kWave * wpr - 1) / (kWave * wpr) > MAX_NV) wpr *= 2;
-        const int nv = (nvec + kWave * wpr - 1) / (kWave * wpr);
-        if (wpr == 1)
-            e = launch_rows_nv<T, 1>(nv, residual, out, bias, gamma, eps, tokens, hidden, flags, s);
-        else if (wpr == 2)
-            e = launch_rows_nv<T, 2>(nv, residual, out, bias, gamma, eps, tokens, hidden, flags, s);
+        while (wpr < kMaxWpr && vectors_per_lane(wpr) > kMaxNv) wpr *= 2;
+        const int nv = vectors_per_lane(wpr);
+        if (tuning(ISP_TUNE_NORM_STORE) != 1)
+            e = launch_rows_wpr<T, true>(wpr, nv, residual, out, bias, gamma, eps, tokens, hidden, flags, s);
         else
-            e = launch_rows_nv<T, 4>(nv, residual, out, bias, gamma, eps, tokens, hidden, flags, s);
+            e = launch_rows_wpr<T, false>(wpr, nv, residual, out, bias, gamma, eps, tokens, hidden, flags, s);
     }
     return note_launch(e);
 }
@@ -202,12 +221,6 @@ static int fused_norm(void* residual_, void* out_, const void* bias_, const void
 }  // namespace isp
 
 extern "C" {
-
-int isp_tuning_norm_waves_per_row(int wpr) {
-    int old = isp::g_norm_wpr;
-    isp::g_norm_wpr = wpr;
-    return old;
-}
 
 int isp_fused_add_bias_residual_rmsnorm_f32(void* residual, void* decoder_out, const void* bias,
                                             const void* gamma, float eps, int tokens, int hidden,

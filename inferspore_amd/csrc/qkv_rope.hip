@@ -10,16 +10,17 @@
 //   v heads and un-rotated elements are copied;  destination [b, head, s, :] of q / k / v.
 //
 // Design (not the reference's one-thread-per-element, one-block-per-(token, head) kernel):
-//   * one 256-thread workgroup per token; the 64 distinct (cos, sin) pairs of that token are
-//     evaluated once by 64 lanes, parked in 512 bytes of LDS and reused by all q and k heads (the
-//     reference evaluates powf + cos + sin again for every head);
-//   * the divisors base^(2d/rot) do not depend on the data, so the host computes them once per
-//     launch configuration with the C library's powf and passes them by value in the kernel
-//     arguments: the device forms angle = t / divisor with one correctly rounded division;
 //   * a lane owns 16 bytes at d = VEC*g and the 16 bytes of the rotation partners at d + hs/2, so
 //     the rotate-half pairing needs no cross-lane exchange, and each group of hs/(2 VEC) lanes
-//     reads and writes whole 128-byte lines of one head row;
-//   * each lane keeps up to UNROLL heads (2 UNROLL vector loads) in flight before computing.
+//     reads and writes whole 128-byte lines of one 256-byte head row;
+//   * a wave carries 8 heads (fp16) of one token; the 64 distinct (cos, sin) pairs of the token are
+//     evaluated once per wave, one pair per lane, and redistributed through 512 bytes of
+//     wave-private LDS (the reference evaluates powf + cos + sin for every (head, d));
+//   * the divisors base^(2d/rot) do not depend on the data, so the host computes them once per
+//     call with the C library's powf and passes them by value in the kernel arguments: the device
+//     forms angle = t / divisor with one correctly rounded division;
+//   * loads are issued before the transcendental work; stores are non-temporal (q, k, v are
+//     consumed by a later kernel, not by this one).
 #include <math.h>
 
 #include "isp_common.h"
@@ -32,104 +33,110 @@ struct RopeDivisors {
     float div[kMaxHalfRot];
 };
 
-template <typename T, int HS, int UNROLL>
-__global__ __launch_bounds__(kBlock) void qkv_rope_vec(
+// A wave owns kWave / G consecutive heads of one token (one head-half pair per lane: two loads and
+// two stores), evaluates the token's (cos, sin) pairs itself (lane d evaluates pair d) and shares
+// them through a wave-private slice of LDS, so there is no workgroup barrier; waves that only carry
+// v heads skip the evaluation.  grid = (tokens, head groups of 4 waves).
+template <typename T, int HS, bool NT>
+__global__ __launch_bounds__(kBlock) void qkv_rope_wave(
     T* __restrict__ q, T* __restrict__ k, T* __restrict__ v, const T* __restrict__ qkv,
     const T* __restrict__ bias, const int32_t* __restrict__ padding_offset,
     const int32_t* __restrict__ history_length, int batch, int seq_len, int head_num,
     int kv_head_num, int half_rot, RopeDivisors tab) {
     constexpr int VEC = Elem<T>::kVec;
     constexpr int HALF = HS / 2;
-    constexpr int G = HALF / VEC;  // lanes per head
-    static_assert(HALF % VEC == 0 && kWave % G == 0, "head size must split into whole lanes");
+    constexpr int G = HALF / VEC;
+    static_assert(HALF % VEC == 0 && kWave % G == 0 && HALF <= kWave, "unsupported head size");
     constexpr int HEADS_PER_WAVE = kWave / G;
-    constexpr int HEADS_PER_PASS = HEADS_PER_WAVE * (kBlock / kWave);
+    constexpr int WAVES = kBlock / kWave;
 
     const int token = blockIdx.x;
     const long long p = (long long)token + (long long)padding_offset[token];
-    if (p < 0 || p >= (long long)batch * (long long)seq_len) return;  // uniform: whole block leaves
+    if (p < 0 || p >= (long long)batch * (long long)seq_len) return;
     const int b = (int)(p / seq_len);
     const int s = (int)(p % seq_len);
-    const int timestep = history_length[b] + s;
-
-    __shared__ float2 cs[HALF];
-    if (threadIdx.x < HALF) {
-        float c = 1.0f, sn = 0.0f;
-        if ((int)threadIdx.x < half_rot) {
-            const float angle = (float)timestep / tab.div[threadIdx.x];
-            sincosf(angle, &sn, &c);
-        }
-        cs[threadIdx.x] = make_float2(c, sn);
-    }
-    __syncthreads();
 
     const int lane = threadIdx.x % kWave;
     const int wave = threadIdx.x / kWave;
     const int g = lane % G;
     const int slot = lane / G;
+    const int qkv_heads = head_num + 2 * kv_head_num;
+    const int wave_first = (blockIdx.y * WAVES + wave) * HEADS_PER_WAVE;
+    if (wave_first >= qkv_heads) return;  // wave-uniform
+    const int h = wave_first + slot;
+    const bool live = h < qkv_heads;
+    const int col = g * VEC;
+    const T* src = qkv + ((size_t)token * (size_t)qkv_heads + (live ? h : 0)) * HS;
+
+    vec16 lo, hi, blo, bhi;
+    if (live) {
+        lo = load16_stream(src + col);
+        hi = load16_stream(src + HALF + col);
+        if (bias) {
+            blo = load16(bias + (size_t)h * HS + col);
+            bhi = load16(bias + (size_t)h * HS + HALF + col);
+        }
+    }
+
     float c[VEC], sn[VEC];
-    bool rot[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; e++) { c[e] = 1.0f; sn[e] = 0.0f; }
+    const bool wave_rotates = wave_first < head_num + kv_head_num;  // wave-uniform
+    if (wave_rotates) {
+        __shared__ float2 cs[WAVES][HALF];
+        if (lane < HALF) {
+            float cc = 1.0f, ss = 0.0f;
+            if (lane < half_rot) {
+                const int timestep = history_length[b] + s;
+                sincosf((float)timestep / tab.div[lane], &ss, &cc);
+            }
+            cs[wave][lane] = make_float2(cc, ss);
+        }
+        // same wave wrote and reads: LDS operations of one wave complete in order
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+        for (int e = 0; e < VEC; e++) {
+            const float2 t = cs[wave][g * VEC + e];
+            c[e] = t.x;
+            sn[e] = t.y;
+        }
+    }
+    if (!live) return;
+
+    float x0[VEC], x1[VEC];
+    Elem<T>::unpack(lo, x0);
+    Elem<T>::unpack(hi, x1);
+    if (bias) {
+        float b0[VEC], b1[VEC];
+        Elem<T>::unpack(blo, b0);
+        Elem<T>::unpack(bhi, b1);
+#pragma unroll
+        for (int e = 0; e < VEC; e++) {
+            x0[e] += b0[e];
+            x1[e] += b1[e];
+        }
+    }
+    T* dst;
+    bool rotate = true;
+    if (h < head_num) {
+        dst = q + (((size_t)b * head_num + h) * seq_len + s) * HS;
+    } else if (h < head_num + kv_head_num) {
+        dst = k + (((size_t)b * kv_head_num + (h - head_num)) * seq_len + s) * HS;
+    } else {
+        dst = v + (((size_t)b * kv_head_num + (h - head_num - kv_head_num)) * seq_len + s) * HS;
+        rotate = false;
+    }
+    float y0[VEC], y1[VEC];
 #pragma unroll
     for (int e = 0; e < VEC; e++) {
-        const float2 t = cs[g * VEC + e];
-        c[e] = t.x;
-        sn[e] = t.y;
-        rot[e] = (g * VEC + e) < half_rot;
+        const bool r = rotate && (g * VEC + e) < half_rot;
+        y0[e] = r ? c[e] * x0[e] - sn[e] * x1[e] : x0[e];
+        y1[e] = r ? c[e] * x1[e] + sn[e] * x0[e] : x1[e];
     }
-
-    const int qkv_heads = head_num + 2 * kv_head_num;
-    const T* row = qkv + (size_t)token * (size_t)qkv_heads * HS;
-    const int col = g * VEC;
-
-    for (int h0 = wave * HEADS_PER_WAVE + slot; h0 < qkv_heads; h0 += HEADS_PER_PASS * UNROLL) {
-        vec16 lo[UNROLL], hi[UNROLL];
-#pragma unroll
-        for (int u = 0; u < UNROLL; u++) {
-            const int h = h0 + u * HEADS_PER_PASS;
-            if (h < qkv_heads) {
-                lo[u] = load16_stream(row + (size_t)h * HS + col);
-                hi[u] = load16_stream(row + (size_t)h * HS + HALF + col);
-            }
-        }
-#pragma unroll
-        for (int u = 0; u < UNROLL; u++) {
-            const int h = h0 + u * HEADS_PER_PASS;
-            if (h < qkv_heads) {
-                float x0[VEC], x1[VEC];
-                Elem<T>::unpack(lo[u], x0);
-                Elem<T>::unpack(hi[u], x1);
-                if (bias) {
-                    float b0[VEC], b1[VEC];
-                    Elem<T>::unpack(load16(bias + (size_t)h * HS + col), b0);
-                    Elem<T>::unpack(load16(bias + (size_t)h * HS + HALF + col), b1);
-#pragma unroll
-                    for (int e = 0; e < VEC; e++) {
-                        x0[e] += b0[e];
-                        x1[e] += b1[e];
-                    }
-                }
-                T* dst;
-                bool rotate = true;
-                if (h < head_num) {
-                    dst = q + (((size_t)b * head_num + h) * seq_len + s) * HS;
-                } else if (h < head_num + kv_head_num) {
-                    dst = k + (((size_t)b * kv_head_num + (h - head_num)) * seq_len + s) * HS;
-                } else {
-                    dst = v + (((size_t)b * kv_head_num + (h - head_num - kv_head_num)) * seq_len + s) * HS;
-                    rotate = false;
-                }
-                float y0[VEC], y1[VEC];
-#pragma unroll
-                for (int e = 0; e < VEC; e++) {
-                    const bool r = rotate && rot[e];
-                    y0[e] = r ? c[e] * x0[e] - sn[e] * x1[e] : x0[e];
-                    y1[e] = r ? c[e] * x1[e] + sn[e] * x0[e] : x1[e];
-                }
-                store16(dst + col, Elem<T>::pack(y0));
-                store16(dst + HALF + col, Elem<T>::pack(y1));
-            }
-        }
-    }
+    store16_sel<NT>(dst + col, Elem<T>::pack(y0));
+    store16_sel<NT>(dst + HALF + col, Elem<T>::pack(y1));
 }
 
 // Any (even) head size and any alignment: one workgroup per token, one lane per rotation pair.
@@ -218,15 +225,24 @@ static int qkv_rope(void* q_, void* k_, void* v_, const void* qkv_, const void* 
                         (!bias || aligned16(bias));
     dim3 grid((unsigned)token_num), block(kBlock);
     hipError_t e;
-    if (vec_ok && head_size == 128) {
-        hipLaunchKernelGGL((qkv_rope_vec<T, 128, 4>), grid, block, 0, s, q, k, v, qkv, bias,
-                           padding_offset, history_length, batch, seq_len, head_num, kv_head_num,
-                           half_rot, tab);
+    const bool nt = tuning(ISP_TUNE_QKV_STORE) != 1;
+#define ISP_QKV_LAUNCH_WAVE(HS)                                                                    \
+    do {                                                                                           \
+        constexpr int HPB = (kWave / ((HS / 2) / Elem<T>::kVec)) * (kBlock / kWave);               \
+        dim3 g2((unsigned)token_num, (unsigned)((head_num + 2 * kv_head_num + HPB - 1) / HPB));    \
+        if (nt) hipLaunchKernelGGL((qkv_rope_wave<T, HS, true>), g2, block, 0, s, q, k, v, qkv, bias, \
+                                   padding_offset, history_length, batch, seq_len, head_num,       \
+                                   kv_head_num, half_rot, tab);                                    \
+        else hipLaunchKernelGGL((qkv_rope_wave<T, HS, false>), g2, block, 0, s, q, k, v, qkv, bias, \
+                                padding_offset, history_length, batch, seq_len, head_num,          \
+                                kv_head_num, half_rot, tab);                                       \
+    } while (0)
+    const int head_groups_max = 65535;
+    if (vec_ok && head_size == 128 && head_num + 2 * kv_head_num <= head_groups_max) {
+        ISP_QKV_LAUNCH_WAVE(128);
         e = hipGetLastError();
-    } else if (vec_ok && head_size == 64) {
-        hipLaunchKernelGGL((qkv_rope_vec<T, 64, 4>), grid, block, 0, s, q, k, v, qkv, bias,
-                           padding_offset, history_length, batch, seq_len, head_num, kv_head_num,
-                           half_rot, tab);
+    } else if (vec_ok && head_size == 64 && head_num + 2 * kv_head_num <= head_groups_max) {
+        ISP_QKV_LAUNCH_WAVE(64);
         e = hipGetLastError();
     } else {
         hipLaunchKernelGGL((qkv_rope_generic<T>), grid, block, 0, s, q, k, v, qkv, bias,

@@ -20,32 +20,47 @@ def f16_ulp_distance(a, b):
     return np.abs(f16_ordered(a) - f16_ordered(b))
 
 
-def assert_f16_close(got, ref, what, max_mismatch_fraction=0.02):
-    """fp16 criterion: every element within 2 ulp of the oracle and within 1e-2 absolute.
+def f16_ulp_size(x):
+    """Spacing of binary16 at magnitude |x| (2^-24 in the subnormal range)."""
+    x = np.abs(np.asarray(x, dtype=np.float64))
+    e = np.floor(np.log2(np.maximum(x, 2.0 ** -14)))
+    return 2.0 ** (e - 10)
+
+
+def assert_f16_close(got, ref, what, magnitude=None, max_mismatch_fraction=0.02):
+    """fp16 criterion: every element within 2 fp16 ulp of the oracle and within 1e-2 absolute.
 
     Where one fp16 ulp is itself larger than 1e-2 (|value| >= 16) a single last-bit rounding
-    difference cannot meet the absolute bound, so there the bound is one ulp.  The share of
-    elements that differ at all is bounded as well, so a systematic error cannot hide in the
-    tolerance."""
+    difference cannot meet the absolute bound, so there the bound is one ulp.
+    `magnitude` (broadcastable to the outputs) is the size of the operands a result was formed
+    from when the result can cancel (a rotation: the radius of the rotated pair).  The fp32
+    arithmetic behind both implementations is only accurate to ~2^-23 of that size, so the ulp is
+    taken at max(|ref|, magnitude / 4096) -- i.e. the bound stays 2 ulp of the value itself unless the
+    value is more than 4096 times smaller than what it was computed from.
+    The share of elements that differ at all is bounded too, so a systematic error cannot hide in
+    the tolerance."""
     got = np.asarray(got)
     ref = np.asarray(ref)
     assert got.dtype == np.float16 and ref.dtype == np.float16, (got.dtype, ref.dtype)
     assert got.shape == ref.shape, (got.shape, ref.shape)
     gnan, rnan = np.isnan(got), np.isnan(ref)
     assert np.array_equal(gnan, rnan), "%s: NaN pattern differs" % what
-    ulp = np.where(rnan, 0, f16_ulp_distance(got, ref))
+    same = (got == ref) | rnan
     with np.errstate(invalid="ignore"):
-        err = np.abs(got.astype(np.float64) - ref.astype(np.float64))
-    err = np.where(rnan | (got == ref), 0.0, err)
+        err = np.where(same, 0.0, np.abs(got.astype(np.float64) - ref.astype(np.float64)))
+    at = np.abs(ref.astype(np.float64))
+    if magnitude is not None:
+        at = np.maximum(at, np.asarray(magnitude, np.float64) / 4096.0)
+    ulp = err / f16_ulp_size(at)
     bad = (ulp > F16_MAX_ULP) | ((err > F16_ATOL) & (ulp > 1))
     if bad.any():
         i = np.unravel_index(np.argmax(bad), bad.shape)
-        raise AssertionError("%s: %d elements out of tolerance; first at %s got %r ref %r (ulp %d)" %
-                             (what, int(bad.sum()), i, got[i], ref[i], int(ulp[i])))
-    frac = float((ulp > 0).mean()) if ulp.size else 0.0
+        raise AssertionError("%s: %d elements out of tolerance; first at %s got %r ref %r (%.2f ulp)" %
+                             (what, int(bad.sum()), i, got[i], ref[i], float(ulp[i])))
+    frac = float((~same).mean()) if same.size else 0.0
     assert frac <= max_mismatch_fraction, "%s: %.3f%% of elements differ from the oracle" % (
         what, 100 * frac)
-    return int(ulp.max()) if ulp.size else 0, frac
+    return (float(ulp.max()) if ulp.size else 0.0), frac
 
 
 def assert_f32_close(got, ref, what, scale=None, rtol=F32_RTOL):
@@ -110,3 +125,15 @@ def qkv_inputs(batch, max_seq, head_num, kv_head_num, head_size, dtype, seed=0, 
     po, _ = padding_offsets_np(lens, max_seq)
     history = np.zeros(batch, np.int32)
     return lens, qkv, bias, po, history
+
+
+def rope_pair_radius(qkv, bias):
+    """[tokens, heads, head_size]: sqrt(x_d^2 + x_{d+half}^2) of the (biased) rotation pair each
+    element belongs to -- the magnitude a rotated output is relative to."""
+    x = np.asarray(qkv, np.float64)
+    hs = x.shape[-1]
+    if bias is not None:
+        x = x + np.asarray(bias, np.float64).reshape(1, -1, hs)
+    half = hs // 2
+    rad = np.sqrt(x[..., :half] ** 2 + x[..., half:] ** 2)
+    return np.concatenate([rad, rad], axis=-1)

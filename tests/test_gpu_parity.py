@@ -6,7 +6,7 @@ import pytest
 import torch
 
 from helpers import (assert_f16_close, assert_f32_close, embedding_inputs, norm_inputs, padding_offsets_np,
-                     qkv_inputs, swiglu_inputs)
+                     qkv_inputs, rope_pair_radius, swiglu_inputs)
 
 pytestmark = pytest.mark.gpu
 
@@ -105,12 +105,12 @@ def _check_norm(isp, oracle, dtype, tokens, hidden, with_res, with_bias, flags=0
     from inferspore_amd import capi
     res, out, bias, gamma = norm_inputs(tokens, hidden, dtype, seed=seed, with_residual=with_res, with_bias=with_bias)
     d_res, d_out = dev(res), dev(out)
-    capi.lib().isp_tuning_norm_waves_per_row(wpr)
+    capi.lib().isp_tuning_set(capi.TUNE_NORM_WAVES_PER_ROW, wpr)
     try:
         isp.fused_add_bias_residual_rmsnorm(d_res, d_out, dev(bias), dev(gamma), 1e-5, flags=flags)
         torch.cuda.synchronize()
     finally:
-        capi.lib().isp_tuning_norm_waves_per_row(0)
+        capi.lib().isp_tuning_set(capi.TUNE_NORM_WAVES_PER_ROW, 0)
     e_res, e_out = oracle.fused_norm(res, out, bias, gamma, 1e-5, flags=flags)
     if dtype == np.float32:
         assert_f32_close(host(d_out), e_out, "normalised output")
@@ -147,7 +147,7 @@ def test_fused_norm_known_answer(isp):
 
 
 @pytest.mark.parametrize("dtype", [np.float16, np.float32])
-@pytest.mark.parametrize("wpr", [0, 1, 2, 4])
+@pytest.mark.parametrize("wpr", [0, 1, 2, 4, 8, 16])
 @pytest.mark.parametrize("tokens,hidden", [(2048, 4096), (7, 4096), (1, 8), (13, 1000), (5, 8192), (3, 11008),
                                            (2, 16384), (9, 520)])
 def test_fused_norm_variants(isp, oracle, dtype, wpr, tokens, hidden):
@@ -255,20 +255,14 @@ def _check_qkv(isp, oracle, dtype, batch, seq, hn, kvn, hs, rot, with_bias=True,
         pad = ~np.broadcast_to(valid[:, None, :, None], exp.shape)
         assert np.array_equal(got[pad], exp[pad]), "padded positions must stay untouched"
     assert np.array_equal(gv, ev), "v is a copy (+ bias in fp32 arithmetic): bit-exact"
-    if dtype == np.float32:
-        x = qkv.astype(np.float64)
-        if bias is not None:
-            x = x + bias.astype(np.float64).reshape(1, -1, hs)
-        half = hs // 2
-        rad = np.sqrt(x[..., :half] ** 2 + x[..., half:] ** 2)
-        rad = np.concatenate([rad, rad], axis=-1)  # [tokens, heads, hs]: the rotation radius of each pair
-        p = np.arange(tokens) + po
-        b, s = p // seq, p % seq
-        for got, exp, sl in ((gq, eq, slice(0, hn)), (gk, ek, slice(hn, hn + kvn))):
+    rad = rope_pair_radius(qkv, bias)
+    p = np.arange(tokens) + po
+    b, s = p // seq, p % seq
+    for got, exp, sl in ((gq, eq, slice(0, hn)), (gk, ek, slice(hn, hn + kvn))):
+        if dtype == np.float32:
             assert_f32_close(got[b, :, s, :], exp[b, :, s, :], "rotated heads", scale=rad[:, sl] + 1e-30)
-    else:
-        assert_f16_close(gq, eq, "q")
-        assert_f16_close(gk, ek, "k")
+        else:
+            assert_f16_close(got[b, :, s, :], exp[b, :, s, :], "rotated heads", magnitude=rad[:, sl])
     return lens
 
 
@@ -328,3 +322,73 @@ def test_qkv_rope_skips_tokens_that_fall_outside(isp):
     isp.add_fused_qkv_bias_transpose_and_rope(q, k, v, qkv, None, po, z, z, 128, 10000.0)
     torch.cuda.synchronize()
     assert torch.all(v[0, :, 0] == 1) and torch.all(v[0, :, 1:] == 0)
+
+
+# ------------------------------------------------------------------ tuning knobs change speed only
+def _with_knobs(settings, fn):
+    from inferspore_amd import capi
+    lib = capi.lib()
+    try:
+        for knob, value in settings.items():
+            assert lib.isp_tuning_set(knob, value) >= 0
+        return fn()
+    finally:
+        for knob in settings:
+            lib.isp_tuning_set(knob, 0)
+
+
+def test_knobs_do_not_change_results(isp):
+    from inferspore_amd import capi
+    import itertools
+    # qkv: every unroll / kernel variant / store kind
+    for dtype in (np.float16, np.float32):
+        lens, qkv, bias, po, hist = qkv_inputs(3, 16, 8, 4, 128, dtype, seed=41, min_len=3)
+        d_in, d_bias, d_po, d_hist, d_lens = dev(qkv), dev(bias), dev(po), dev(hist), dev(lens)
+
+        def run_qkv():
+            outs = [torch.full((3, n, 16, 128), -3, dtype=NP2T[dtype], device="cuda") for n in (8, 4, 4)]
+            isp.add_fused_qkv_bias_transpose_and_rope(outs[0], outs[1], outs[2], d_in, d_bias, d_po, d_hist, d_lens,
+                                                      128, 10000.0)
+            return [host(o) for o in outs]
+
+        base = run_qkv()
+        for store in (1, 2):
+            say("qkv knobs %s store=%d" % (dtype.__name__, store))
+            got = _with_knobs({capi.TUNE_QKV_STORE: store}, run_qkv)
+            assert all(np.array_equal(a, b) for a, b in zip(got, base))
+    # embedding
+    ids, table = embedding_inputs(77, 4096, 300, np.float16, seed=43)
+    d_ids, d_table = dev(ids), dev(table)
+
+    def run_embed():
+        out = torch.zeros((77, 4096), dtype=torch.float16, device="cuda")
+        isp.input_embedding(d_ids, out, d_table)
+        return host(out)
+
+    base = run_embed()
+    for variant, store in itertools.product((1, 2, 3), (1, 2)):
+        say("embedding knobs variant=%d store=%d" % (variant, store))
+        assert np.array_equal(_with_knobs({capi.TUNE_EMBED_VARIANT: variant, capi.TUNE_EMBED_STORE: store}, run_embed), base)
+    # swiglu
+    x = dev(swiglu_inputs(19, 11008, np.float16, seed=47))
+
+    def run_swiglu():
+        out = torch.zeros((19, 11008), dtype=torch.float16, device="cuda")
+        isp.act(x, out)
+        return host(out)
+
+    base = run_swiglu()
+    for unroll, store in itertools.product((1, 2, 4), (1, 2)):
+        assert np.array_equal(_with_knobs({capi.TUNE_SWIGLU_UNROLL: unroll, capi.TUNE_SWIGLU_STORE: store}, run_swiglu), base)
+    # norm: store kind (waves per row is swept against the oracle above)
+    res, out, bias, gamma = norm_inputs(50, 4096, np.float16, seed=53)
+
+    def run_norm():
+        d_res, d_out = dev(res), dev(out)
+        isp.fused_add_bias_residual_rmsnorm(d_res, d_out, dev(bias), dev(gamma), 1e-5)
+        return host(d_res), host(d_out)
+
+    base = run_norm()
+    for store in (1, 2):
+        got = _with_knobs({capi.TUNE_NORM_STORE: store}, run_norm)
+        assert np.array_equal(got[0], base[0]) and np.array_equal(got[1], base[1])
