@@ -28,6 +28,21 @@ import time
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published peak
 
+# HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE and WRITE_SIZE in separate runs, each
+# scaled by what the same counter reads for isp_calibration_copy of known size: x1.9984 and x1.0000).
+# The summary of those runs is profiles/all_kernels_llama7b_shapes.hbm_traffic_pmc.txt.
+MEASURED_TRAFFIC_BYTES = {
+    "fused_add_bias_residual_rmsnorm_f16_2048x4096": 67261704,
+    "rmsnorm_f32_64x4096": 2257998,
+    "rmsnorm_f32_16384x4096": 536838689,
+    "embedding_f16_8192x4096_v32000": 133718151,
+    "qkv_bias_rope_transpose_f16_b8_s512": 146727112,
+    "swiglu_f16_prefill_8192x11008": 540815334,
+    "swiglu_f16_decode_256x11008": 16928129,
+    "calibration_copy_64MiB_traffic": 67108864,
+    "calibration_copy_512MiB_traffic": 536685713,
+}
+
 
 def parse():
     ap = argparse.ArgumentParser()
@@ -242,7 +257,7 @@ def measure(torch, w, steps, warmup, stream):
         "GBps": gbs, "frac_of_hbm_peak": gbs / HBM_PEAK_GBS,
         "tokens_per_s": (w.tokens / (event_ms * 1e-3)) if w.tokens else None,
         "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": gbs / HBM_PEAK_GBS, "traffic": None},
+                     "frac": gbs / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC_BYTES.get(w.name)},
     }
 
 
