@@ -197,7 +197,7 @@ def make_workloads(torch, lib, stream_handle, rotate):
         # calibration: a plain copy with the same traffic as the headline workload
         w = Workload()
         w.name, w.dtype, w.tokens = "calibration_copy_%dMiB_traffic" % (2 * nbytes >> 20), "u8", 0
-        w.kernel = "isp::copy_vec<4>"
+        w.kernel = "isp::copy_vec<1>"
         w.bytes_per_launch = 2 * nbytes
         R = w.sets_for(2 * nbytes, rotate)
         srcs = [torch.empty(nbytes, device=dev, dtype=torch.uint8).fill_(j & 255) for j in range(R)]

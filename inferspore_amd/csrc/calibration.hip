@@ -1,6 +1,7 @@
 // A plain device-to-device copy of known size.  It has no counterpart in the reference: it exists so
 // that profiler byte counters (and the achievable copy bandwidth of the machine) can be calibrated
-// against a kernel whose traffic is known exactly -- `bytes` read and `bytes` written.
+// against a kernel whose traffic is known exactly -- `bytes` read and `bytes` written.  It uses the
+// same access recipe as the production kernels (16-byte vectors, one per lane, non-temporal).
 #include "isp_common.h"
 
 namespace isp {
@@ -18,7 +19,7 @@ __global__ __launch_bounds__(kBlock) void copy_vec(char* __restrict__ dst,
 #pragma unroll
     for (int k = 0; k < UNROLL; k++) {
         const size_t v = first + (size_t)k * kBlock;
-        if (v < nvec) store16(dst + v * 16, buf[k]);
+        if (v < nvec) store16_stream(dst + v * 16, buf[k]);
     }
 }
 
@@ -29,7 +30,7 @@ extern "C" int isp_calibration_copy(void* dst, const void* src, size_t bytes, is
     ISP_REQUIRE_PTR(dst);
     ISP_REQUIRE_PTR(src);
     if (bytes % 16 != 0 || !isp::aligned16(dst) || !isp::aligned16(src)) return ISP_ERR_BAD_SHAPE;
-    constexpr int UNROLL = 4;
+    constexpr int UNROLL = 1;  // one vector per lane streams best on this memory system
     const size_t nvec = bytes / 16;
     const size_t per_block = (size_t)isp::kBlock * UNROLL;
     const size_t blocks = (nvec + per_block - 1) / per_block;

@@ -50,18 +50,21 @@ __global__ __launch_bounds__(kBlock) void qkv_rope_wave(
     constexpr int HEADS_PER_WAVE = kWave / G;
     constexpr int WAVES = kBlock / kWave;
 
-    const int token = blockIdx.x;
+    // grid = (tokens, head groups): the token index runs fastest, so the workgroups in flight at any
+    // time read 8 KiB slices of consecutive token rows and write into one group of 32 heads
+    // (measured: faster than token-major order and than 4-token workgroups).
+    const int lane = threadIdx.x % kWave;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const int token = (int)blockIdx.x;
     const long long p = (long long)token + (long long)padding_offset[token];
-    if (p < 0 || p >= (long long)batch * (long long)seq_len) return;
+    if (p < 0 || p >= (long long)batch * (long long)seq_len) return;  // wave-uniform
     const int b = (int)(p / seq_len);
     const int s = (int)(p % seq_len);
 
-    const int lane = threadIdx.x % kWave;
-    const int wave = threadIdx.x / kWave;
     const int g = lane % G;
     const int slot = lane / G;
     const int qkv_heads = head_num + 2 * kv_head_num;
-    const int wave_first = (blockIdx.y * WAVES + wave) * HEADS_PER_WAVE;
+    const int wave_first = ((int)blockIdx.y * WAVES + wave) * HEADS_PER_WAVE;
     if (wave_first >= qkv_heads) return;  // wave-uniform
     const int h = wave_first + slot;
     const bool live = h < qkv_heads;
@@ -226,18 +229,17 @@ static int qkv_rope(void* q_, void* k_, void* v_, const void* qkv_, const void* 
     dim3 grid((unsigned)token_num), block(kBlock);
     hipError_t e;
     const bool nt = tuning(ISP_TUNE_QKV_STORE) != 1;
+#define ISP_QKV_LAUNCH_1(HS, N, GRID)                                                              \
+    hipLaunchKernelGGL((qkv_rope_wave<T, HS, N>), GRID, block, 0, s, q, k, v, qkv, bias,            \
+                       padding_offset, history_length, batch, seq_len, head_num, kv_head_num,      \
+                       half_rot, tab)
 #define ISP_QKV_LAUNCH_WAVE(HS)                                                                    \
     do {                                                                                           \
         constexpr int HPB = (kWave / ((HS / 2) / Elem<T>::kVec)) * (kBlock / kWave);               \
         dim3 g2((unsigned)token_num, (unsigned)((head_num + 2 * kv_head_num + HPB - 1) / HPB));    \
-        if (nt) hipLaunchKernelGGL((qkv_rope_wave<T, HS, true>), g2, block, 0, s, q, k, v, qkv, bias, \
-                                   padding_offset, history_length, batch, seq_len, head_num,       \
-                                   kv_head_num, half_rot, tab);                                    \
-        else hipLaunchKernelGGL((qkv_rope_wave<T, HS, false>), g2, block, 0, s, q, k, v, qkv, bias, \
-                                padding_offset, history_length, batch, seq_len, head_num,          \
-                                kv_head_num, half_rot, tab);                                       \
+        if (nt) ISP_QKV_LAUNCH_1(HS, true, g2); else ISP_QKV_LAUNCH_1(HS, false, g2);              \
     } while (0)
-    const int head_groups_max = 65535;
+    const int head_groups_max = 65535 * 4;  // grid.y limit, 4 heads per workgroup at least
     if (vec_ok && head_size == 128 && head_num + 2 * kv_head_num <= head_groups_max) {
         ISP_QKV_LAUNCH_WAVE(128);
         e = hipGetLastError();
