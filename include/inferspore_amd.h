@@ -142,6 +142,64 @@ int isp_swiglu_f32(const void* in, void* out, int tokens, int inter, isp_stream_
 int isp_swiglu_f16(const void* in, void* out, int tokens, int inter, isp_stream_t stream);
 
 /*
+ * Decode-phase RoPE, in place: rotate-half on the q and k heads of packed rows
+ * [batch, head_num + 2 kv_head_num, head_size] at timestep step - 1.
+ * Replaces launchRoPE<T> (src/kernels/qkv_bias_and_RoPE.h:22-25, .cu:352-434; the reference's fp16
+ * body is empty and its launcher only accepts batch 1, 32+32+32 heads of 128).
+ */
+int isp_rope_decode_f32(void* qkv, int batch, int head_num, int kv_head_num, int head_size, int step,
+                        int rotary_embedding_dim, float rotary_embedding_base, isp_stream_t stream);
+int isp_rope_decode_f16(void* qkv, int batch, int head_num, int kv_head_num, int head_size, int step,
+                        int rotary_embedding_dim, float rotary_embedding_base, isp_stream_t stream);
+
+/*
+ * Transpose attention output and remove padding: dst[t, h, :] = src[b, h, s, :] with
+ * t + padding_offset[t] = b * seq_len + s.  src [batch, head_num, seq_len, head_size],
+ * dst [token_num, head_num, head_size].
+ * Supplies launchTransposeOutRemovePadding<T>, which the reference declares
+ * (src/kernels/fused_transpose_and_remv_pad.h:7-10) and tests
+ * (tests/unittests/test_fused_trans_remv_pad.cu) but does not define.
+ */
+int isp_transpose_remove_padding_f32(const void* src, const int32_t* padding_offset, void* dst,
+                                     int batch, int head_num, int seq_len, int head_size,
+                                     int token_num, isp_stream_t stream);
+int isp_transpose_remove_padding_f16(const void* src, const int32_t* padding_offset, void* dst,
+                                     int batch, int head_num, int seq_len, int head_size,
+                                     int token_num, isp_stream_t stream);
+
+/*
+ * KV-cache append: cache[layer][b, h, history_length[b] + t, :] = src[b, h, t, :] for
+ * t < cur_query_length[b], for k and v in one launch.
+ * k_src, v_src [batch, kv_head_num, max_q_len, head_size];
+ * k_cache, v_cache [layers, batch, kv_head_num, max_seq_len, head_size] (base pointers; `layer`
+ * selects the slice).  Replaces launchConcatKVCache<T> (src/kernels/concat_past_kv.h:7-14,
+ * .cu:7-113).
+ */
+int isp_concat_kv_cache_f32(const void* k_src, const void* v_src, void* k_cache, void* v_cache,
+                            int layer, const int32_t* cur_query_length,
+                            const int32_t* history_length, int batch, int kv_head_num, int max_q_len,
+                            int max_seq_len, int head_size, isp_stream_t stream);
+int isp_concat_kv_cache_f16(const void* k_src, const void* v_src, void* k_cache, void* v_cache,
+                            int layer, const int32_t* cur_query_length,
+                            const int32_t* history_length, int batch, int kv_head_num, int max_q_len,
+                            int max_seq_len, int head_size, isp_stream_t stream);
+
+/*
+ * KV-cache broadcast to the query heads (GQA / MQA):
+ * dst[b, h, s, :] = cache[layer][b, h / (head_num / kv_head_num), s, :] for s < context_length[b].
+ * k_dst, v_dst [batch, head_num, max_k_len, head_size].
+ * Replaces launchRepeatKVCache<T> (src/kernels/repeat_kv.h:7-13, .cu:10-100).
+ */
+int isp_repeat_kv_cache_f32(const void* k_cache, const void* v_cache, void* k_dst, void* v_dst,
+                            int layer, const int32_t* context_length, int batch, int head_num,
+                            int kv_head_num, int max_seq_len, int max_k_len, int head_size,
+                            isp_stream_t stream);
+int isp_repeat_kv_cache_f16(const void* k_cache, const void* v_cache, void* k_dst, void* v_dst,
+                            int layer, const int32_t* context_length, int batch, int head_num,
+                            int kv_head_num, int max_seq_len, int max_k_len, int head_size,
+                            isp_stream_t stream);
+
+/*
  * Measurement aids (no reference counterpart).
  * isp_calibration_copy: a plain copy kernel of known traffic (`bytes` read + `bytes` written;
  *   16-byte aligned, multiple of 16) used to calibrate profiler byte counters and to measure the

@@ -15,3 +15,10 @@ void launchAddFusedQKVBiasTransposeAndRoPE(TensorWrapper<T>* q_buf, TensorWrappe
                                            TensorWrapper<int>* history_length,
                                            TensorWrapper<int>* input_length,
                                            LLaMAAttentionStaticParams& params);
+
+// launchRoPE -- same declaration as the reference's src/kernels/qkv_bias_and_RoPE.h:22-25 (decode
+// phase): in-place rotate-half RoPE on qkv_buf [1, 96, 128] at timestep step - 1; `step` is a host
+// (CPU) tensor.  The reference's checks (batch 1, 96 heads of 128, 32 q heads) are kept.
+template <typename T>
+void launchRoPE(TensorWrapper<T>* qkv_buf, TensorWrapper<int>* step,
+                LLaMAAttentionStaticParams& static_params);

@@ -34,6 +34,14 @@ SIGNATURES = {
     "isp_qkv_bias_rope_transpose_f16": (_i, [_vp] * 8 + [_i] * 7 + [_f, _i, _i, _vp]),
     "isp_swiglu_f32": (_i, [_vp, _vp, _i, _i, _vp]),
     "isp_swiglu_f16": (_i, [_vp, _vp, _i, _i, _vp]),
+    "isp_rope_decode_f32": (_i, [_vp, _i, _i, _i, _i, _i, _i, _f, _vp]),
+    "isp_rope_decode_f16": (_i, [_vp, _i, _i, _i, _i, _i, _i, _f, _vp]),
+    "isp_transpose_remove_padding_f32": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
+    "isp_transpose_remove_padding_f16": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
+    "isp_concat_kv_cache_f32": (_i, [_vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
+    "isp_concat_kv_cache_f16": (_i, [_vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
+    "isp_repeat_kv_cache_f32": (_i, [_vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i, _i, _i, _vp]),
+    "isp_repeat_kv_cache_f16": (_i, [_vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i, _i, _i, _vp]),
     "isp_tuning_set": (_i, [_i, _i]),
     "isp_calibration_copy": (_i, [_vp, _vp, C.c_size_t, _vp]),
 }

@@ -94,17 +94,25 @@ struct Elem<__half> {
             f[2 * i + 1] = p.y;
         }
     }
+    // The fp32 value is pinned in a register before the conversion.  Without that the compiler may
+    // merge the producing multiply-add with the conversion into one mixed-precision instruction
+    // that rounds the exact product-sum straight to fp16; kernels would then differ from each other
+    // (and from "fp32 arithmetic, one rounding of the fp32 result") on rounding ties.
+    __device__ static __forceinline__ float pinned(float x) {
+        asm volatile("" : "+v"(x));
+        return x;
+    }
     __device__ static __forceinline__ vec16 pack(const float* f) {
         vec16 v;
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            __half2 h = __floats2half2_rn(f[2 * i], f[2 * i + 1]);
+            __half2 h = __floats2half2_rn(pinned(f[2 * i]), pinned(f[2 * i + 1]));
             v.w[i] = *reinterpret_cast<const uint32_t*>(&h);
         }
         return v;
     }
     __device__ static __forceinline__ float to_f32(__half x) { return __half2float(x); }
-    __device__ static __forceinline__ __half from_f32(float x) { return __float2half_rn(x); }
+    __device__ static __forceinline__ __half from_f32(float x) { return __float2half_rn(pinned(x)); }
 };
 
 // DPP lane exchange inside the VALU (no LDS traffic).  `ctrl` is the DPP control word.

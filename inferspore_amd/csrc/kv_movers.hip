@@ -1,0 +1,268 @@
+// The strided copies either side of attention, for gfx950: transpose-out + remove padding, KV-cache
+// append, KV-cache broadcast.  All three move whole head rows (head_size elements), so they are
+// written once on bytes and serve every element type bit-exactly.
+//
+//   transpose_remove_padding   [batch, heads, seq, hs] -> [tokens, heads, hs]
+//       contract: src/kernels/fused_transpose_and_remv_pad.h:7-10 and
+//       tests/unittests/test_fused_trans_remv_pad.cu:3,28-49 (the reference declares and tests this
+//       launcher but holds no definition); it is the inverse of the QKV scatter
+//       (src/kernels/qkv_bias_and_RoPE.cu:135-140).
+//   concat_kv_cache            src/kernels/concat_past_kv.cu:7-113
+//   repeat_kv_cache            src/kernels/repeat_kv.cu:10-100
+//
+// Design: one 16-byte vector per lane, a workgroup covers one 4 KiB chunk of the contiguous side,
+// non-temporal stores; k and v go in one launch (the reference issues two).  Rows whose index
+// would fall outside the destination are skipped instead of written out of bounds.
+#include "isp_common.h"
+
+namespace isp {
+
+// dst[token, h, :] = src[b, h, s, :],  token + padding_offset[token] = b * seq_len + s.
+// grid = tokens * chunks, a chunk being 256 vectors of the token's heads*seg_vec vectors
+__global__ __launch_bounds__(kBlock) void transpose_remove_padding_vec(
+    const char* __restrict__ src, const int32_t* __restrict__ padding_offset, char* __restrict__ dst,
+    int batch, int head_num, int seq_len, unsigned seg_vec, unsigned chunks) {
+    const unsigned token = blockIdx.x / chunks;
+    const unsigned vi = (blockIdx.x % chunks) * kBlock + threadIdx.x;  // vector index inside the token's row
+    const unsigned row_vec = (unsigned)head_num * seg_vec;
+    if (vi >= row_vec) return;
+    const long long p = (long long)token + (long long)padding_offset[token];
+    if (p < 0 || p >= (long long)batch * seq_len) return;
+    const unsigned b = (unsigned)(p / seq_len), s = (unsigned)(p % seq_len);
+    const unsigned h = vi / seg_vec, c = vi % seg_vec;
+    const size_t from = ((((size_t)b * head_num + h) * seq_len + s) * seg_vec + c) * 16u;
+    store16_stream(dst + ((size_t)token * row_vec + vi) * 16u, load16_stream(src + from));
+}
+
+__global__ __launch_bounds__(kBlock) void transpose_remove_padding_bytes(
+    const char* src, const int32_t* padding_offset, char* dst, int batch, int head_num, int seq_len,
+    size_t seg_bytes) {
+    const unsigned token = blockIdx.x;
+    const long long p = (long long)token + (long long)padding_offset[token];
+    if (p < 0 || p >= (long long)batch * seq_len) return;
+    const size_t b = (size_t)(p / seq_len), s = (size_t)(p % seq_len);
+    const size_t row = (size_t)head_num * seg_bytes;
+    for (size_t i = threadIdx.x; i < row; i += kBlock) {
+        const size_t h = i / seg_bytes, c = i % seg_bytes;
+        dst[(size_t)token * row + i] = src[((b * head_num + h) * seq_len + s) * seg_bytes + c];
+    }
+}
+
+// cache[b, h, history[b] + t, :] = src[b, h, t, :] for t < cur_len[b]; blockIdx.z selects k / v.
+// grid = (chunks of max_q_len*seg_vec vectors, batch * kv_heads, 2)
+__global__ __launch_bounds__(kBlock) void concat_kv_vec(
+    const char* __restrict__ k_src, const char* __restrict__ v_src, char* __restrict__ k_cache,
+    char* __restrict__ v_cache, const int32_t* __restrict__ cur_query_length,
+    const int32_t* __restrict__ history_length, int kv_head_num, int max_q_len, int max_seq_len,
+    unsigned seg_vec) {
+    const char* src = blockIdx.z == 0 ? k_src : v_src;
+    char* cache = blockIdx.z == 0 ? k_cache : v_cache;
+    const unsigned bh = blockIdx.y;
+    const unsigned b = bh / kv_head_num;
+    const unsigned vi = blockIdx.x * kBlock + threadIdx.x;
+    if (vi >= (unsigned)max_q_len * seg_vec) return;
+    const unsigned t = vi / seg_vec, c = vi % seg_vec;
+    const int cur = cur_query_length[b];
+    const long long row = (long long)history_length[b] + t;
+    if ((int)t >= cur || row < 0 || row >= max_seq_len) return;
+    store16_stream(cache + (((size_t)bh * max_seq_len + (size_t)row) * seg_vec + c) * 16u,
+                   load16_stream(src + ((size_t)bh * max_q_len * seg_vec + vi) * 16u));
+}
+
+__global__ __launch_bounds__(kBlock) void concat_kv_bytes(
+    const char* k_src, const char* v_src, char* k_cache, char* v_cache,
+    const int32_t* cur_query_length, const int32_t* history_length, int kv_head_num, int max_q_len,
+    int max_seq_len, size_t seg_bytes) {
+    const char* src = blockIdx.z == 0 ? k_src : v_src;
+    char* cache = blockIdx.z == 0 ? k_cache : v_cache;
+    const unsigned bh = blockIdx.y, b = bh / kv_head_num, t = blockIdx.x;
+    const long long row = (long long)history_length[b] + t;
+    if ((int)t >= cur_query_length[b] || row < 0 || row >= max_seq_len) return;
+    for (size_t i = threadIdx.x; i < seg_bytes; i += kBlock)
+        cache[((size_t)bh * max_seq_len + (size_t)row) * seg_bytes + i] =
+            src[((size_t)bh * max_q_len + t) * seg_bytes + i];
+}
+
+// dst[b, h, s, :] = cache[b, h / rep, s, :] for s < context_length[b]; blockIdx.z selects k / v.
+// grid = (chunks of max_k_len*seg_vec vectors, batch * heads, 2)
+__global__ __launch_bounds__(kBlock) void repeat_kv_vec(
+    const char* __restrict__ k_cache, const char* __restrict__ v_cache, char* __restrict__ k_dst,
+    char* __restrict__ v_dst, const int32_t* __restrict__ context_length, int head_num,
+    int kv_head_num, int max_seq_len, int max_k_len, unsigned seg_vec) {
+    const char* cache = blockIdx.z == 0 ? k_cache : v_cache;
+    char* dst = blockIdx.z == 0 ? k_dst : v_dst;
+    const unsigned bh = blockIdx.y;
+    const unsigned b = bh / head_num, h = bh % head_num;
+    const unsigned vi = blockIdx.x * kBlock + threadIdx.x;
+    if (vi >= (unsigned)max_k_len * seg_vec) return;
+    const unsigned s = vi / seg_vec;
+    if ((int)s >= context_length[b] || (int)s >= max_seq_len) return;
+    const unsigned kvh = h / (unsigned)(head_num / kv_head_num);
+    store16_stream(dst + ((size_t)bh * max_k_len * seg_vec + vi) * 16u,
+                   load16_stream(cache + (((size_t)b * kv_head_num + kvh) * max_seq_len * seg_vec + vi) * 16u));
+}
+
+__global__ __launch_bounds__(kBlock) void repeat_kv_bytes(
+    const char* k_cache, const char* v_cache, char* k_dst, char* v_dst,
+    const int32_t* context_length, int head_num, int kv_head_num, int max_seq_len, int max_k_len,
+    size_t seg_bytes) {
+    const char* cache = blockIdx.z == 0 ? k_cache : v_cache;
+    char* dst = blockIdx.z == 0 ? k_dst : v_dst;
+    const unsigned bh = blockIdx.y, b = bh / head_num, h = bh % head_num, s = blockIdx.x;
+    if ((int)s >= context_length[b] || (int)s >= max_seq_len) return;
+    const unsigned kvh = h / (unsigned)(head_num / kv_head_num);
+    for (size_t i = threadIdx.x; i < seg_bytes; i += kBlock)
+        dst[((size_t)bh * max_k_len + s) * seg_bytes + i] =
+            cache[(((size_t)b * kv_head_num + kvh) * max_seq_len + s) * seg_bytes + i];
+}
+
+constexpr long long kMaxGridYZ = 65535;
+
+static int transpose_remove_padding(const void* src, const int32_t* padding_offset, void* dst,
+                                    int batch, int head_num, int seq_len, int head_size,
+                                    int token_num, int elem, hipStream_t s) {
+    if (batch < 0 || head_num < 0 || seq_len < 0 || head_size < 0 || token_num < 0) return ISP_ERR_BAD_SHAPE;
+    if (token_num == 0 || head_num == 0 || head_size == 0) return ISP_OK;
+    if (batch == 0 || seq_len == 0) return ISP_ERR_BAD_SHAPE;
+    ISP_REQUIRE_PTR(src);
+    ISP_REQUIRE_PTR(padding_offset);
+    ISP_REQUIRE_PTR(dst);
+    const size_t seg = (size_t)head_size * elem;
+    const size_t chunks = ((size_t)head_num * (seg / 16) + kBlock - 1) / kBlock;
+    if (seg % 16 == 0 && aligned16(src) && aligned16(dst) && chunks * (size_t)token_num <= 0x7fffffffull) {
+        const unsigned seg_vec = (unsigned)(seg / 16);
+        dim3 grid((unsigned)(chunks * (size_t)token_num));
+        hipLaunchKernelGGL(transpose_remove_padding_vec, grid, dim3(kBlock), 0, s,
+                           static_cast<const char*>(src), padding_offset, static_cast<char*>(dst),
+                           batch, head_num, seq_len, seg_vec, (unsigned)chunks);
+    } else {
+        hipLaunchKernelGGL(transpose_remove_padding_bytes, dim3((unsigned)token_num), dim3(kBlock), 0,
+                           s, static_cast<const char*>(src), padding_offset, static_cast<char*>(dst),
+                           batch, head_num, seq_len, seg);
+    }
+    return note_launch(hipGetLastError());
+}
+
+static int concat_kv(const void* k_src, const void* v_src, void* k_cache, void* v_cache, int layer,
+                     const int32_t* cur_query_length, const int32_t* history_length, int batch,
+                     int kv_head_num, int max_q_len, int max_seq_len, int head_size, int elem,
+                     hipStream_t s) {
+    if (batch < 0 || kv_head_num < 0 || max_q_len < 0 || max_seq_len < 0 || head_size < 0 || layer < 0)
+        return ISP_ERR_BAD_SHAPE;
+    if (batch == 0 || kv_head_num == 0 || max_q_len == 0 || head_size == 0) return ISP_OK;
+    ISP_REQUIRE_PTR(k_src);
+    ISP_REQUIRE_PTR(v_src);
+    ISP_REQUIRE_PTR(k_cache);
+    ISP_REQUIRE_PTR(v_cache);
+    ISP_REQUIRE_PTR(cur_query_length);
+    ISP_REQUIRE_PTR(history_length);
+    if ((long long)batch * kv_head_num > kMaxGridYZ) return ISP_ERR_UNSUPPORTED;
+    const size_t seg = (size_t)head_size * elem;
+    // layer offset = layer * batch * kv_head_num * max_seq_len * head_size elements (concat_past_kv.cu:89)
+    const size_t layer_bytes = (size_t)layer * batch * kv_head_num * max_seq_len * seg;
+    char* kc = static_cast<char*>(k_cache) + layer_bytes;
+    char* vc = static_cast<char*>(v_cache) + layer_bytes;
+    const char* ks = static_cast<const char*>(k_src);
+    const char* vs = static_cast<const char*>(v_src);
+    if (seg % 16 == 0 && aligned16(ks) && aligned16(vs) && aligned16(kc) && aligned16(vc)) {
+        const unsigned seg_vec = (unsigned)(seg / 16);
+        const size_t row_vec = (size_t)max_q_len * seg_vec;
+        if (row_vec > 0xffffffffull) return ISP_ERR_UNSUPPORTED;
+        dim3 grid((unsigned)((row_vec + kBlock - 1) / kBlock), (unsigned)(batch * kv_head_num), 2);
+        hipLaunchKernelGGL(concat_kv_vec, grid, dim3(kBlock), 0, s, ks, vs, kc, vc, cur_query_length,
+                           history_length, kv_head_num, max_q_len, max_seq_len, seg_vec);
+    } else {
+        dim3 grid((unsigned)max_q_len, (unsigned)(batch * kv_head_num), 2);
+        hipLaunchKernelGGL(concat_kv_bytes, grid, dim3(kBlock), 0, s, ks, vs, kc, vc, cur_query_length,
+                           history_length, kv_head_num, max_q_len, max_seq_len, seg);
+    }
+    return note_launch(hipGetLastError());
+}
+
+static int repeat_kv(const void* k_cache, const void* v_cache, void* k_dst, void* v_dst, int layer,
+                     const int32_t* context_length, int batch, int head_num, int kv_head_num,
+                     int max_seq_len, int max_k_len, int head_size, int elem, hipStream_t s) {
+    if (batch < 0 || head_num < 0 || kv_head_num < 0 || max_seq_len < 0 || max_k_len < 0 ||
+        head_size < 0 || layer < 0)
+        return ISP_ERR_BAD_SHAPE;
+    if (batch == 0 || head_num == 0 || max_k_len == 0 || head_size == 0) return ISP_OK;
+    if (kv_head_num == 0 || head_num % kv_head_num != 0) return ISP_ERR_BAD_SHAPE;
+    ISP_REQUIRE_PTR(k_cache);
+    ISP_REQUIRE_PTR(v_cache);
+    ISP_REQUIRE_PTR(k_dst);
+    ISP_REQUIRE_PTR(v_dst);
+    ISP_REQUIRE_PTR(context_length);
+    if ((long long)batch * head_num > kMaxGridYZ) return ISP_ERR_UNSUPPORTED;
+    const size_t seg = (size_t)head_size * elem;
+    const size_t layer_bytes = (size_t)layer * batch * kv_head_num * max_seq_len * seg;  // repeat_kv.cu:70
+    const char* kc = static_cast<const char*>(k_cache) + layer_bytes;
+    const char* vc = static_cast<const char*>(v_cache) + layer_bytes;
+    char* kd = static_cast<char*>(k_dst);
+    char* vd = static_cast<char*>(v_dst);
+    if (seg % 16 == 0 && aligned16(kc) && aligned16(vc) && aligned16(kd) && aligned16(vd)) {
+        const unsigned seg_vec = (unsigned)(seg / 16);
+        const size_t row_vec = (size_t)max_k_len * seg_vec;
+        if (row_vec > 0xffffffffull) return ISP_ERR_UNSUPPORTED;
+        dim3 grid((unsigned)((row_vec + kBlock - 1) / kBlock), (unsigned)(batch * head_num), 2);
+        hipLaunchKernelGGL(repeat_kv_vec, grid, dim3(kBlock), 0, s, kc, vc, kd, vd, context_length,
+                           head_num, kv_head_num, max_seq_len, max_k_len, seg_vec);
+    } else {
+        dim3 grid((unsigned)max_k_len, (unsigned)(batch * head_num), 2);
+        hipLaunchKernelGGL(repeat_kv_bytes, grid, dim3(kBlock), 0, s, kc, vc, kd, vd, context_length,
+                           head_num, kv_head_num, max_seq_len, max_k_len, seg);
+    }
+    return note_launch(hipGetLastError());
+}
+
+}  // namespace isp
+
+extern "C" {
+
+int isp_transpose_remove_padding_f32(const void* src, const int32_t* padding_offset, void* dst,
+                                     int batch, int head_num, int seq_len, int head_size,
+                                     int token_num, isp_stream_t stream) {
+    return isp::transpose_remove_padding(src, padding_offset, dst, batch, head_num, seq_len, head_size,
+                                         token_num, 4, static_cast<hipStream_t>(stream));
+}
+int isp_transpose_remove_padding_f16(const void* src, const int32_t* padding_offset, void* dst,
+                                     int batch, int head_num, int seq_len, int head_size,
+                                     int token_num, isp_stream_t stream) {
+    return isp::transpose_remove_padding(src, padding_offset, dst, batch, head_num, seq_len, head_size,
+                                         token_num, 2, static_cast<hipStream_t>(stream));
+}
+
+int isp_concat_kv_cache_f32(const void* k_src, const void* v_src, void* k_cache, void* v_cache,
+                            int layer, const int32_t* cur_query_length,
+                            const int32_t* history_length, int batch, int kv_head_num, int max_q_len,
+                            int max_seq_len, int head_size, isp_stream_t stream) {
+    return isp::concat_kv(k_src, v_src, k_cache, v_cache, layer, cur_query_length, history_length,
+                          batch, kv_head_num, max_q_len, max_seq_len, head_size, 4,
+                          static_cast<hipStream_t>(stream));
+}
+int isp_concat_kv_cache_f16(const void* k_src, const void* v_src, void* k_cache, void* v_cache,
+                            int layer, const int32_t* cur_query_length,
+                            const int32_t* history_length, int batch, int kv_head_num, int max_q_len,
+                            int max_seq_len, int head_size, isp_stream_t stream) {
+    return isp::concat_kv(k_src, v_src, k_cache, v_cache, layer, cur_query_length, history_length,
+                          batch, kv_head_num, max_q_len, max_seq_len, head_size, 2,
+                          static_cast<hipStream_t>(stream));
+}
+
+int isp_repeat_kv_cache_f32(const void* k_cache, const void* v_cache, void* k_dst, void* v_dst,
+                            int layer, const int32_t* context_length, int batch, int head_num,
+                            int kv_head_num, int max_seq_len, int max_k_len, int head_size,
+                            isp_stream_t stream) {
+    return isp::repeat_kv(k_cache, v_cache, k_dst, v_dst, layer, context_length, batch, head_num,
+                          kv_head_num, max_seq_len, max_k_len, head_size, 4,
+                          static_cast<hipStream_t>(stream));
+}
+int isp_repeat_kv_cache_f16(const void* k_cache, const void* v_cache, void* k_dst, void* v_dst,
+                            int layer, const int32_t* context_length, int batch, int head_num,
+                            int kv_head_num, int max_seq_len, int max_k_len, int head_size,
+                            isp_stream_t stream) {
+    return isp::repeat_kv(k_cache, v_cache, k_dst, v_dst, layer, context_length, batch, head_num,
+                          kv_head_num, max_seq_len, max_k_len, head_size, 2,
+                          static_cast<hipStream_t>(stream));
+}
+
+}  // extern "C"

@@ -6,9 +6,12 @@
 #include "inferspore_amd.h"
 #include "src/kernels/act_kernel.h"
 #include "src/kernels/cal_paddingoffset.h"
+#include "src/kernels/concat_past_kv.h"
 #include "src/kernels/fused_addresidual_norm.h"
+#include "src/kernels/fused_transpose_and_remv_pad.h"
 #include "src/kernels/input_embedding.h"
 #include "src/kernels/qkv_bias_and_RoPE.h"
+#include "src/kernels/repeat_kv.h"
 #include "src/kernels/rmsnorm.h"
 
 namespace {
@@ -22,6 +25,10 @@ struct Abi<float> {
     static constexpr auto fused_norm = isp_fused_add_bias_residual_rmsnorm_f32;
     static constexpr auto qkv = isp_qkv_bias_rope_transpose_f32;
     static constexpr auto swiglu = isp_swiglu_f32;
+    static constexpr auto rope_decode = isp_rope_decode_f32;
+    static constexpr auto transpose_remove_padding = isp_transpose_remove_padding_f32;
+    static constexpr auto concat_kv = isp_concat_kv_cache_f32;
+    static constexpr auto repeat_kv = isp_repeat_kv_cache_f32;
 };
 template <>
 struct Abi<half> {
@@ -30,6 +37,10 @@ struct Abi<half> {
     static constexpr auto fused_norm = isp_fused_add_bias_residual_rmsnorm_f16;
     static constexpr auto qkv = isp_qkv_bias_rope_transpose_f16;
     static constexpr auto swiglu = isp_swiglu_f16;
+    static constexpr auto rope_decode = isp_rope_decode_f16;
+    static constexpr auto transpose_remove_padding = isp_transpose_remove_padding_f16;
+    static constexpr auto concat_kv = isp_concat_kv_cache_f16;
+    static constexpr auto repeat_kv = isp_repeat_kv_cache_f16;
 };
 
 inline void expect_ok(int status, const char* what) {
@@ -118,6 +129,74 @@ void launchAct(TensorWrapper<T>* input, TensorWrapper<T>* out) {
     expect_ok(Abi<T>::swiglu(input->data, out->data, tokens, inter, nullptr), "launchAct");
 }
 
+// reference: src/kernels/qkv_bias_and_RoPE.cu:404-434 (hard-wired to LLaMA-7B: 32 q heads, batch 1)
+template <typename T>
+void launchRoPE(TensorWrapper<T>* qkv_buf, TensorWrapper<int>* step,
+                LLaMAAttentionStaticParams& static_params) {
+    const int batch_size = qkv_buf->shape[0];
+    const int qkv_head_num = qkv_buf->shape[1];
+    const int head_num = 32;
+    const int head_size = qkv_buf->shape[2];
+    LLM_CHECK(batch_size == 1);
+    LLM_CHECK(qkv_head_num == 96);
+    LLM_CHECK(head_size == 128);
+    const int cur_step = step->getVal();
+    expect_ok(Abi<T>::rope_decode(qkv_buf->data, batch_size, head_num, head_num, head_size, cur_step,
+                                  static_params.rotary_embedding_dim,
+                                  static_params.rotary_embedding_base, nullptr),
+              "launchRoPE");
+}
+
+// contract: src/kernels/fused_transpose_and_remv_pad.h:7-10, tests/unittests/test_fused_trans_remv_pad.cu:40-49
+template <typename T>
+void launchTransposeOutRemovePadding(TensorWrapper<T>* qkv_buf_w_pad, TensorWrapper<int>* padding_offset,
+                                     TensorWrapper<T>* qkv_buf_wo_pad_1) {
+    const int batch_size = qkv_buf_w_pad->shape[0];
+    const int head_num = qkv_buf_w_pad->shape[1];
+    const int seq_len = qkv_buf_w_pad->shape[2];
+    const int head_size = qkv_buf_w_pad->shape[3];
+    const int token_num = qkv_buf_wo_pad_1->shape[0];
+    expect_ok(Abi<T>::transpose_remove_padding(qkv_buf_w_pad->data, padding_offset->data,
+                                               qkv_buf_wo_pad_1->data, batch_size, head_num, seq_len,
+                                               head_size, token_num, nullptr),
+              "launchTransposeOutRemovePadding");
+}
+
+// reference: src/kernels/concat_past_kv.cu:76-113 (shape derivation :84-90)
+template <typename T>
+void launchConcatKVCache(TensorWrapper<T>* k_src, TensorWrapper<T>* v_src, TensorWrapper<int>* layer_id,
+                         TensorWrapper<int>* cur_query_length, TensorWrapper<int>* history_length,
+                         TensorWrapper<T>* k_dst, TensorWrapper<T>* v_dst) {
+    const int batch_size = k_src->shape[0];
+    const int max_seq_len = k_dst->shape[3];
+    const int kv_head_num = k_src->shape[1];
+    const int max_q_len = k_src->shape[2];
+    const int head_size = k_src->shape[3];
+    const int layer = layer_id->getVal();
+    expect_ok(Abi<T>::concat_kv(k_src->data, v_src->data, k_dst->data, v_dst->data, layer,
+                                cur_query_length->data, history_length->data, batch_size, kv_head_num,
+                                max_q_len, max_seq_len, head_size, nullptr),
+              "launchConcatKVCache");
+}
+
+// reference: src/kernels/repeat_kv.cu:52-100 (shape derivation :59-70)
+template <typename T>
+void launchRepeatKVCache(TensorWrapper<T>* k_cache_src, TensorWrapper<T>* v_cache_src,
+                         TensorWrapper<int>* context_length, TensorWrapper<int>* layer_id,
+                         TensorWrapper<T>* k_cache_dst, TensorWrapper<T>* v_cache_dst) {
+    const int batch_size = context_length->shape[0];
+    const int kv_head_num = k_cache_src->shape[2];
+    const int max_seq_len = k_cache_src->shape[3];
+    const int head_num = k_cache_dst->shape[1];
+    const int max_k_len = k_cache_dst->shape[2];
+    const int head_size = k_cache_dst->shape[3];
+    const int layer = layer_id->getVal();
+    expect_ok(Abi<T>::repeat_kv(k_cache_src->data, v_cache_src->data, k_cache_dst->data,
+                                v_cache_dst->data, layer, context_length->data, batch_size, head_num,
+                                kv_head_num, max_seq_len, max_k_len, head_size, nullptr),
+              "launchRepeatKVCache");
+}
+
 // explicit instantiations for float and half, as in the reference
 #define ISP_INSTANTIATE(T)                                                                          \
     template void launchInputEmbedding(TensorWrapper<int>*, TensorWrapper<T>*, EmbeddingWeight<T>*); \
@@ -127,7 +206,15 @@ void launchAct(TensorWrapper<T>* input, TensorWrapper<T>* out) {
     template void launchAddFusedQKVBiasTransposeAndRoPE(                                            \
         TensorWrapper<T>*, TensorWrapper<T>*, TensorWrapper<T>*, TensorWrapper<T>*, BaseWeight<T>&, \
         TensorWrapper<int>*, TensorWrapper<int>*, TensorWrapper<int>*, LLaMAAttentionStaticParams&); \
-    template void launchAct(TensorWrapper<T>*, TensorWrapper<T>*);
+    template void launchAct(TensorWrapper<T>*, TensorWrapper<T>*);                                  \
+    template void launchRoPE(TensorWrapper<T>*, TensorWrapper<int>*, LLaMAAttentionStaticParams&);  \
+    template void launchTransposeOutRemovePadding(TensorWrapper<T>*, TensorWrapper<int>*,           \
+                                                  TensorWrapper<T>*);                               \
+    template void launchConcatKVCache(TensorWrapper<T>*, TensorWrapper<T>*, TensorWrapper<int>*,    \
+                                      TensorWrapper<int>*, TensorWrapper<int>*, TensorWrapper<T>*,  \
+                                      TensorWrapper<T>*);                                           \
+    template void launchRepeatKVCache(TensorWrapper<T>*, TensorWrapper<T>*, TensorWrapper<int>*,    \
+                                      TensorWrapper<int>*, TensorWrapper<T>*, TensorWrapper<T>*);
 ISP_INSTANTIATE(float)
 ISP_INSTANTIATE(half)
 #undef ISP_INSTANTIATE

@@ -33,6 +33,23 @@ struct RopeDivisors {
     float div[kMaxHalfRot];
 };
 
+// (cos, sin) of timestep / divisor.  Kept out of line so that the prefill, decode and scalar kernels
+// all execute the very same instruction sequence: a decode step at `step` and a prefill token at
+// history = step - 1 then produce identical bits.
+__device__ __attribute__((noinline)) float2 rope_coefficients(int timestep, float divisor) {
+    float sn, c;
+    sincosf((float)timestep / divisor, &sn, &c);
+    return make_float2(c, sn);
+}
+
+// One rotation, with the contraction spelled out so that every kernel in this file rounds the same
+// way: y0 = c x0 - s x1, y1 = c x1 + s x0, each as one product plus one fused multiply-add.
+__device__ __forceinline__ void rotate_pair(float c, float sn, float x0, float x1, float& y0,
+                                            float& y1) {
+    y0 = __fmaf_rn(c, x0, -(sn * x1));
+    y1 = __fmaf_rn(c, x1, sn * x0);
+}
+
 // A wave owns kWave / G consecutive heads of one token (one head-half pair per lane: two loads and
 // two stores), evaluates the token's (cos, sin) pairs itself (lane d evaluates pair d) and shares
 // them through a wave-private slice of LDS, so there is no workgroup barrier; waves that only carry
@@ -88,12 +105,9 @@ __global__ __launch_bounds__(kBlock) void qkv_rope_wave(
     if (wave_rotates) {
         __shared__ float2 cs[WAVES][HALF];
         if (lane < HALF) {
-            float cc = 1.0f, ss = 0.0f;
-            if (lane < half_rot) {
-                const int timestep = history_length[b] + s;
-                sincosf((float)timestep / tab.div[lane], &ss, &cc);
-            }
-            cs[wave][lane] = make_float2(cc, ss);
+            float2 coef = make_float2(1.0f, 0.0f);
+            if (lane < half_rot) coef = rope_coefficients(history_length[b] + s, tab.div[lane]);
+            cs[wave][lane] = coef;
         }
         // same wave wrote and reads: LDS operations of one wave complete in order
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -135,8 +149,10 @@ __global__ __launch_bounds__(kBlock) void qkv_rope_wave(
 #pragma unroll
     for (int e = 0; e < VEC; e++) {
         const bool r = rotate && (g * VEC + e) < half_rot;
-        y0[e] = r ? c[e] * x0[e] - sn[e] * x1[e] : x0[e];
-        y1[e] = r ? c[e] * x1[e] + sn[e] * x0[e] : x1[e];
+        float r0, r1;
+        rotate_pair(c[e], sn[e], x0[e], x1[e], r0, r1);
+        y0[e] = r ? r0 : x0[e];
+        y1[e] = r ? r1 : x1[e];
     }
     store16_sel<NT>(dst + col, Elem<T>::pack(y0));
     store16_sel<NT>(dst + HALF + col, Elem<T>::pack(y1));
@@ -179,14 +195,123 @@ __global__ __launch_bounds__(kBlock) void qkv_rope_generic(
         }
         float y0 = x0, y1 = x1;
         if (rotate) {
-            float c, sn;
-            sincosf((float)timestep / tab.div[d], &sn, &c);
-            y0 = c * x0 - sn * x1;
-            y1 = c * x1 + sn * x0;
+            const float2 coef = rope_coefficients(timestep, tab.div[d]);
+            rotate_pair(coef.x, coef.y, x0, x1, y0, y1);
         }
         dst[d] = Elem<T>::from_f32(y0);
         dst[half + d] = Elem<T>::from_f32(y1);
     }
+}
+
+// Decode-phase RoPE, in place on packed rows [batch, head_num + 2 kv_head_num, head_size]
+// (src/kernels/qkv_bias_and_RoPE.cu:352-390, launcher :404-434): rotate-half on every q and k head
+// at timestep step - 1 (:380).  Same lane layout as the prefill kernel: a wave owns kWave / G heads of
+// one row, evaluates the 64 (cos, sin) pairs once and shares them through wave-private LDS.
+// Each k head is rotated once (the reference rotates k head q / (head_num / kv_head_num) from every q
+// block, which only coincides with this when kv_head_num == head_num, the one case it accepts).
+template <typename T, int HS>
+__global__ __launch_bounds__(kBlock) void rope_decode_wave(T* __restrict__ qkv, int head_num,
+                                                           int kv_head_num, int timestep,
+                                                           int half_rot, RopeDivisors tab) {
+    constexpr int VEC = Elem<T>::kVec;
+    constexpr int HALF = HS / 2;
+    constexpr int G = HALF / VEC;
+    constexpr int HEADS_PER_WAVE = kWave / G;
+    constexpr int WAVES = kBlock / kWave;
+    const int lane = threadIdx.x % kWave;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const int g = lane % G;
+    const int slot = lane / G;
+    const int rotated_heads = head_num + kv_head_num;
+    const int wave_first = ((int)blockIdx.y * WAVES + wave) * HEADS_PER_WAVE;
+    if (wave_first >= rotated_heads) return;  // wave-uniform
+    const int h = wave_first + slot;
+    const bool live = h < rotated_heads;
+    T* p = qkv + ((size_t)blockIdx.x * (size_t)(head_num + 2 * kv_head_num) + (live ? h : 0)) * HS + g * VEC;
+    vec16 lo, hi;
+    if (live) {
+        lo = load16(p);
+        hi = load16(p + HALF);
+    }
+    __shared__ float2 cs[WAVES][HALF];
+    if (lane < HALF) {
+        float2 coef = make_float2(1.0f, 0.0f);
+        if (lane < half_rot) coef = rope_coefficients(timestep, tab.div[lane]);
+        cs[wave][lane] = coef;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    if (!live) return;
+    float x0[VEC], x1[VEC], y0[VEC], y1[VEC];
+    Elem<T>::unpack(lo, x0);
+    Elem<T>::unpack(hi, x1);
+#pragma unroll
+    for (int e = 0; e < VEC; e++) {
+        const float2 t = cs[wave][g * VEC + e];
+        const bool r = (g * VEC + e) < half_rot;
+        float r0, r1;
+        rotate_pair(t.x, t.y, x0[e], x1[e], r0, r1);
+        y0[e] = r ? r0 : x0[e];
+        y1[e] = r ? r1 : x1[e];
+    }
+    store16(p, Elem<T>::pack(y0));
+    store16(p + HALF, Elem<T>::pack(y1));
+}
+
+template <typename T>
+__global__ __launch_bounds__(kBlock) void rope_decode_generic(T* qkv, int head_num, int kv_head_num,
+                                                              int head_size, int timestep,
+                                                              int half_rot, RopeDivisors tab) {
+    const int half = head_size / 2;
+    T* row = qkv + (size_t)blockIdx.x * (size_t)(head_num + 2 * kv_head_num) * head_size;
+    const int pairs = (head_num + kv_head_num) * half_rot;
+    for (int i = threadIdx.x; i < pairs; i += kBlock) {
+        const int h = i / half_rot, d = i % half_rot;
+        T* p = row + (size_t)h * head_size + d;
+        const float x0 = Elem<T>::to_f32(p[0]), x1 = Elem<T>::to_f32(p[half]);
+        float y0, y1;
+        const float2 coef = rope_coefficients(timestep, tab.div[d]);
+        rotate_pair(coef.x, coef.y, x0, x1, y0, y1);
+        p[0] = Elem<T>::from_f32(y0);
+        p[half] = Elem<T>::from_f32(y1);
+    }
+}
+
+static void fill_divisors(RopeDivisors& tab, int rot, float base) {
+    const int half_rot = rot / 2;
+    for (int d = 0; d < kMaxHalfRot; d++)
+        tab.div[d] = d < half_rot ? powf(base, (float)(2 * d) / (float)rot) : 1.0f;
+}
+
+template <typename T>
+static int rope_decode(void* qkv_, int batch, int head_num, int kv_head_num, int head_size, int step,
+                       int rot, float base, hipStream_t s) {
+    if (batch < 0 || head_num < 0 || kv_head_num < 0 || head_size < 0 || rot < 0) return ISP_ERR_BAD_SHAPE;
+    if (batch == 0 || head_size == 0 || head_num + kv_head_num == 0 || rot == 0) return ISP_OK;
+    if (head_size % 2 != 0 || rot % 2 != 0 || rot > head_size) return ISP_ERR_BAD_SHAPE;
+    if (rot / 2 > kMaxHalfRot) return ISP_ERR_UNSUPPORTED;
+    ISP_REQUIRE_PTR(qkv_);
+    T* qkv = static_cast<T*>(qkv_);
+    RopeDivisors tab;
+    fill_divisors(tab, rot, base);
+    const int timestep = step - 1;  // qkv_bias_and_RoPE.cu:380
+    const int half_rot = rot / 2;
+    dim3 block(kBlock);
+    if (aligned16(qkv) && (head_size == 128 || head_size == 64) && head_num + kv_head_num <= 65535) {
+        const int hpb = (kWave / ((head_size / 2) / Elem<T>::kVec)) * (kBlock / kWave);
+        dim3 grid((unsigned)batch, (unsigned)((head_num + kv_head_num + hpb - 1) / hpb));
+        if (head_size == 128)
+            hipLaunchKernelGGL((rope_decode_wave<T, 128>), grid, block, 0, s, qkv, head_num, kv_head_num,
+                               timestep, half_rot, tab);
+        else
+            hipLaunchKernelGGL((rope_decode_wave<T, 64>), grid, block, 0, s, qkv, head_num, kv_head_num,
+                               timestep, half_rot, tab);
+    } else {
+        hipLaunchKernelGGL((rope_decode_generic<T>), dim3((unsigned)batch), block, 0, s, qkv, head_num,
+                           kv_head_num, head_size, timestep, half_rot, tab);
+    }
+    return note_launch(hipGetLastError());
 }
 
 template <typename T>
@@ -221,8 +346,7 @@ static int qkv_rope(void* q_, void* k_, void* v_, const void* qkv_, const void* 
 
     RopeDivisors tab;
     const int half_rot = rot / 2;
-    for (int d = 0; d < kMaxHalfRot; d++)
-        tab.div[d] = d < half_rot ? powf(base, (float)(2 * d) / (float)rot) : 1.0f;
+    fill_divisors(tab, rot, base);
 
     const bool vec_ok = aligned16(q) && aligned16(k) && aligned16(v) && aligned16(qkv) &&
                         (!bias || aligned16(bias));
@@ -287,6 +411,20 @@ int isp_qkv_bias_rope_transpose_f16(void* q, void* k, void* v, const void* qkv, 
                                  batch, seq_len, token_num, head_num, kv_head_num, head_size,
                                  rotary_embedding_dim, rotary_embedding_base,
                                  static_cast<hipStream_t>(stream));
+}
+
+int isp_rope_decode_f32(void* qkv, int batch, int head_num, int kv_head_num, int head_size, int step,
+                        int rotary_embedding_dim, float rotary_embedding_base, isp_stream_t stream) {
+    return isp::rope_decode<float>(qkv, batch, head_num, kv_head_num, head_size, step,
+                                   rotary_embedding_dim, rotary_embedding_base,
+                                   static_cast<hipStream_t>(stream));
+}
+
+int isp_rope_decode_f16(void* qkv, int batch, int head_num, int kv_head_num, int head_size, int step,
+                        int rotary_embedding_dim, float rotary_embedding_base, isp_stream_t stream) {
+    return isp::rope_decode<__half>(qkv, batch, head_num, kv_head_num, head_size, step,
+                                    rotary_embedding_dim, rotary_embedding_base,
+                                    static_cast<hipStream_t>(stream));
 }
 
 }  // extern "C"

@@ -114,3 +114,51 @@ def act(input, out):
     fn = getattr(capi.lib(), "isp_swiglu_" + _suffix(input))
     capi.check(fn(_p(input), _p(out), input.shape[0], input.shape[2], _stream()), "isp_swiglu")
     return out
+
+
+def rope(qkv_buf, step, head_num, rotary_embedding_dim, rotary_embedding_base):
+    """launchRoPE (decode): in place on qkv_buf [batch, head_num + 2 kv_head_num, head_size]; `step` is a
+    host integer (the reference reads it from a CPU tensor)."""
+    _dev(qkv_buf)
+    batch, qkv_head_num, head_size = qkv_buf.shape
+    kv_head_num = (qkv_head_num - head_num) // 2
+    fn = getattr(capi.lib(), "isp_rope_decode_" + _suffix(qkv_buf))
+    capi.check(fn(_p(qkv_buf), batch, head_num, kv_head_num, head_size, int(step), int(rotary_embedding_dim),
+                  float(rotary_embedding_base), _stream()), "isp_rope_decode")
+    return qkv_buf
+
+
+def transpose_out_remove_padding(qkv_buf_w_pad, padding_offset, qkv_buf_wo_pad):
+    """launchTransposeOutRemovePadding: [batch, heads, seq, hs] -> [tokens, heads, hs]."""
+    _dev(qkv_buf_w_pad, padding_offset, qkv_buf_wo_pad)
+    batch, head_num, seq_len, head_size = qkv_buf_w_pad.shape
+    token_num = qkv_buf_wo_pad.shape[0]
+    fn = getattr(capi.lib(), "isp_transpose_remove_padding_" + _suffix(qkv_buf_w_pad))
+    capi.check(fn(_p(qkv_buf_w_pad), _p(padding_offset), _p(qkv_buf_wo_pad), batch, head_num, seq_len, head_size,
+                  token_num, _stream()), "isp_transpose_remove_padding")
+    return qkv_buf_wo_pad
+
+
+def concat_kv_cache(k_src, v_src, layer_id, cur_query_length, history_length, k_dst, v_dst):
+    """launchConcatKVCache; shapes as the reference derives them (concat_past_kv.cu:84-90)."""
+    _dev(k_src, v_src, cur_query_length, history_length, k_dst, v_dst)
+    batch, kv_head_num, max_q_len, head_size = k_src.shape
+    max_seq_len = k_dst.shape[3]
+    fn = getattr(capi.lib(), "isp_concat_kv_cache_" + _suffix(k_src))
+    capi.check(fn(_p(k_src), _p(v_src), _p(k_dst), _p(v_dst), int(layer_id), _p(cur_query_length),
+                  _p(history_length), batch, kv_head_num, max_q_len, max_seq_len, head_size, _stream()),
+               "isp_concat_kv_cache")
+    return k_dst, v_dst
+
+
+def repeat_kv_cache(k_cache_src, v_cache_src, context_length, layer_id, k_cache_dst, v_cache_dst):
+    """launchRepeatKVCache; shapes as the reference derives them (repeat_kv.cu:59-70)."""
+    _dev(k_cache_src, v_cache_src, context_length, k_cache_dst, v_cache_dst)
+    batch = context_length.shape[0]
+    kv_head_num, max_seq_len = k_cache_src.shape[2], k_cache_src.shape[3]
+    head_num, max_k_len, head_size = k_cache_dst.shape[1], k_cache_dst.shape[2], k_cache_dst.shape[3]
+    fn = getattr(capi.lib(), "isp_repeat_kv_cache_" + _suffix(k_cache_src))
+    capi.check(fn(_p(k_cache_src), _p(v_cache_src), _p(k_cache_dst), _p(v_cache_dst), int(layer_id),
+                  _p(context_length), batch, head_num, kv_head_num, max_seq_len, max_k_len, head_size, _stream()),
+               "isp_repeat_kv_cache")
+    return k_cache_dst, v_cache_dst

@@ -23,12 +23,26 @@ def test_launch_api_case(case):
     assert "passed" in p.stdout
 
 
+NEIGHBOURS = os.path.join(ROOT, "build", "bin", "test_launch_neighbours")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("case", ["rope", "transpose", "kvcache"])
+def test_launch_neighbours_case(case):
+    assert os.path.exists(NEIGHBOURS), "build/bin/test_launch_neighbours is missing: run python -m inferspore_amd.build"
+    print("[case] test_launch_neighbours " + case, flush=True)
+    p = subprocess.run([NEIGHBOURS, case], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=100)
+    assert p.returncode == 0, p.stdout[-3000:]
+    assert "passed" in p.stdout
+
+
 def test_launch_library_exports_all_instantiations():
     assert os.path.exists(LAUNCH_LIB), "libinferspore_launch.so is missing: run python -m inferspore_amd.build"
     syms = subprocess.run(["nm", "-D", "--defined-only", "-C", LAUNCH_LIB], stdout=subprocess.PIPE, text=True,
                           check=True).stdout
     for name in ("launchInputEmbedding", "launchFusedAddBiasResidualRMSNorm", "launchRMSNorm",
-                 "launchAddFusedQKVBiasTransposeAndRoPE", "launchAct"):
+                 "launchAddFusedQKVBiasTransposeAndRoPE", "launchAct", "launchRoPE",
+                 "launchTransposeOutRemovePadding", "launchConcatKVCache", "launchRepeatKVCache"):
         for t in ("float", "__half"):
             assert any(name + "<" + t + ">" in line for line in syms.splitlines()), (name, t)
     assert "launchCalPaddingoffset(" in syms
