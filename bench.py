@@ -193,6 +193,77 @@ def make_workloads(torch, lib, stream_handle, rotate):
         w.config = {"tokens": tokens, "inter": inter}
         return w
 
+    def padded_batch():
+        batch, seq = 8, 512
+        g = torch.Generator(device="cpu").manual_seed(0)
+        lens = torch.randint(256, 513, (batch,), generator=g, dtype=torch.int32)
+        lens_d = lens.to(dev)
+        po = torch.zeros((batch, seq), device=dev, dtype=torch.int32)
+        cum = torch.zeros((batch + 1,), device=dev, dtype=torch.int32)
+        assert lib.isp_cal_padding_offset(po.data_ptr(), cum.data_ptr(), lens_d.data_ptr(), batch, seq, st) == 0
+        return batch, seq, int(lens.sum()), lens_d, po
+
+    def transpose_out():
+        w = Workload()
+        batch, seq, tokens, lens_d, po = padded_batch()
+        hn, hs = 32, 128
+        w.name, w.dtype, w.tokens = "transpose_remove_padding_f16_b8_s512", "f16", tokens
+        w.kernel = "isp::transpose_remove_padding_vec"
+        w.bytes_per_launch = tokens * (2 * hn * hs * 2 + 4)
+        R = w.sets_for(batch * hn * seq * hs * 2 + tokens * hn * hs * 2, rotate)
+        srcs = [torch.randn((batch, hn, seq, hs), device=dev).to(torch.float16) for _ in range(R)]
+        dsts = [torch.empty((tokens, hn, hs), device=dev, dtype=torch.float16) for _ in range(R)]
+        w.keep = (lens_d, po, srcs, dsts)
+        w.bind(lib.isp_transpose_remove_padding_f16,
+               [(srcs[j].data_ptr(), po.data_ptr(), dsts[j].data_ptr(), batch, hn, seq, hs, tokens, st)
+                for j in range(R)])
+        w.reset = lambda: None
+        w.config = {"batch": batch, "max_seq": seq, "valid_tokens": tokens, "heads": hn, "head_dim": hs}
+        return w
+
+    def kv_cache(which):
+        w = Workload()
+        batch, seq, tokens, lens_d, po = padded_batch()
+        kvn, hn, hs, max_seq, layers = 32, 32, 128, 1024, 1
+        hist = torch.zeros(batch, device=dev, dtype=torch.int32)
+        # append: read + write k and v rows of the valid tokens; broadcast: same volume with MHA (rep = 1)
+        w.bytes_per_launch = 2 * 2 * tokens * kvn * hs * 2 + 2 * batch * 4
+        w.dtype, w.tokens = "f16", tokens
+        R = w.sets_for(2 * batch * kvn * (seq + max_seq) * hs * 2, rotate)
+        smalls = [[torch.randn((batch, kvn, seq, hs), device=dev).to(torch.float16) for _ in range(2)] for _ in range(R)]
+        caches = [[torch.zeros((layers, batch, kvn, max_seq, hs), device=dev, dtype=torch.float16) for _ in range(2)]
+                  for _ in range(R)]
+        w.keep = (lens_d, po, hist, smalls, caches)
+        if which == "append":
+            w.name, w.kernel = "concat_kv_cache_f16_b8_q512_S1024", "isp::concat_kv_vec"
+            w.bind(lib.isp_concat_kv_cache_f16,
+                   [(smalls[j][0].data_ptr(), smalls[j][1].data_ptr(), caches[j][0].data_ptr(),
+                     caches[j][1].data_ptr(), 0, lens_d.data_ptr(), hist.data_ptr(), batch, kvn, seq, max_seq, hs, st)
+                    for j in range(R)])
+        else:
+            w.name, w.kernel = "repeat_kv_cache_f16_b8_k512_S1024", "isp::repeat_kv_vec"
+            w.bind(lib.isp_repeat_kv_cache_f16,
+                   [(caches[j][0].data_ptr(), caches[j][1].data_ptr(), smalls[j][0].data_ptr(),
+                     smalls[j][1].data_ptr(), 0, lens_d.data_ptr(), batch, hn, kvn, max_seq, seq, hs, st)
+                    for j in range(R)])
+        w.reset = lambda: None
+        w.config = {"batch": batch, "max_q_len": seq, "max_seq_len": max_seq, "valid_tokens": tokens,
+                    "kv_heads": kvn, "head_dim": hs}
+        return w
+
+    def rope_decode():
+        w = Workload()
+        w.name, w.dtype, w.tokens = "rope_decode_f16_1x96x128", "f16", 1
+        w.kernel = "isp::rope_decode_wave<__half, 128>"
+        w.bytes_per_launch = 2 * 64 * 128 * 2
+        R = 64 if rotate else 1
+        rows = [torch.randn((1, 96, 128), device=dev).to(torch.float16) for _ in range(R)]
+        w.keep = rows
+        w.bind(lib.isp_rope_decode_f16, [(rows[j].data_ptr(), 1, 32, 32, 128, 17, 128, 10000.0, st) for j in range(R)])
+        w.reset = lambda: None
+        w.config = {"batch": 1, "heads": "32q/32kv", "head_dim": 128}
+        return w
+
     def copy(nbytes):
         # calibration: a plain copy with the same traffic as the headline workload
         w = Workload()
@@ -217,6 +288,10 @@ def make_workloads(torch, lib, stream_handle, rotate):
         ("qkv_bias_rope_transpose_f16_b8_s512", qkv),
         ("swiglu_f16_prefill_8192x11008", lambda: swiglu(8192, "prefill")),
         ("swiglu_f16_decode_256x11008", lambda: swiglu(256, "decode")),
+        ("transpose_remove_padding_f16_b8_s512", transpose_out),
+        ("concat_kv_cache_f16_b8_q512_S1024", lambda: kv_cache("append")),
+        ("repeat_kv_cache_f16_b8_k512_S1024", lambda: kv_cache("broadcast")),
+        ("rope_decode_f16_1x96x128", rope_decode),
         ("calibration_copy_64MiB_traffic", lambda: copy(32 << 20)),
         ("calibration_copy_512MiB_traffic", lambda: copy(256 << 20)),
     ]
