@@ -1,0 +1,81 @@
+"""The entry points allocate nothing, synchronise nothing and record only kernel nodes, so a caller
+can capture a launch-bound sequence of them into a HIP graph.  A decode-step-like sequence is captured
+once and replayed several times, with eager work and synchronisation between replays; every replay
+must reproduce the eager results bit for bit."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def _sequence(isp, t):
+    """One decode step's worth of the memory-bound kernels on pre-allocated tensors (batch of 16)."""
+    isp.fused_add_bias_residual_rmsnorm(t["residual"], t["hidden"], None, t["gamma"], 1e-5)
+    isp.rope(t["qkv"], t["step"], 32, 128, 10000.0)
+    isp.concat_kv_cache(t["k_new"], t["v_new"], 0, t["cur"], t["hist"], t["k_cache"], t["v_cache"])
+    isp.repeat_kv_cache(t["k_cache"], t["v_cache"], t["ctx"], 0, t["k_rep"], t["v_rep"])
+    isp.act(t["gate_up"], t["act_out"])
+    isp.rmsnorm(t["hidden"], t["gamma"], 1e-5)
+
+
+def _tensors(seed):
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    r = lambda *s: torch.randn(s, device="cuda", generator=g).half()
+    batch, kvn, hn, hs, max_seq = 16, 8, 32, 128, 64
+    return {
+        "hidden": r(batch, 4096), "residual": r(batch, 4096), "gamma": r(4096),
+        "qkv": r(1, 96, 128), "step": 9,
+        "k_new": r(batch, kvn, 1, hs), "v_new": r(batch, kvn, 1, hs),
+        "cur": torch.ones(batch, dtype=torch.int32, device="cuda"),
+        "hist": torch.full((batch,), 8, dtype=torch.int32, device="cuda"),
+        "ctx": torch.full((batch,), 9, dtype=torch.int32, device="cuda"),
+        "k_cache": r(1, batch, kvn, max_seq, hs), "v_cache": r(1, batch, kvn, max_seq, hs),
+        "k_rep": torch.zeros((batch, hn, 9, hs), dtype=torch.float16, device="cuda"),
+        "v_rep": torch.zeros((batch, hn, 9, hs), dtype=torch.float16, device="cuda"),
+        "gate_up": r(batch, 2, 11008), "act_out": torch.zeros((batch, 11008), dtype=torch.float16, device="cuda"),
+    }
+
+
+def _snapshot(t):
+    return {k: v.clone() for k, v in t.items() if torch.is_tensor(v)}
+
+
+def test_capture_and_replay_matches_eager(isp):
+    print("[case] graph capture of a decode-step sequence", flush=True)
+    t = _tensors(1)
+    initial = _snapshot(t)
+    # eager reference: three steps in a row (the in-place kernels make each step depend on the last)
+    eager = []
+    for _ in range(3):
+        _sequence(isp, t)
+        torch.cuda.synchronize()
+        eager.append(_snapshot(t))
+    # restore, capture one step
+    for k, v in initial.items():
+        t[k].copy_(v)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        # warm-up on the capture stream (outside the capture), then restore the state
+        _sequence(isp, t)
+        for k, v in initial.items():
+            t[k].copy_(v)
+        side.synchronize()
+        graph.capture_begin()
+        _sequence(isp, t)      # ops.* launch on torch's current stream, which is the capturing one
+        graph.capture_end()
+    torch.cuda.synchronize()
+    for k, v in initial.items():   # capture does not execute: the state is still the initial one
+        assert torch.equal(t[k], v), k
+    scratch = torch.zeros(1 << 20, device="cuda")
+    for step in range(3):
+        graph.replay()
+        torch.cuda.synchronize()
+        for k, v in eager[step].items():
+            assert torch.equal(t[k], v), "replay %d differs from eager in %s" % (step, k)
+        # unrelated eager work and a synchronisation between replays
+        scratch.add_(1.0)
+        isp.rmsnorm(torch.randn((4, 4096), device="cuda").half(), t["gamma"], 1e-5)
+        torch.cuda.synchronize()
