@@ -29,18 +29,22 @@ import time
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published peak
 
 # HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE and WRITE_SIZE in separate runs, each
-# scaled by what the same counter reads for isp_calibration_copy of known size: x1.9984 and x1.0000).
-# The summary of those runs is profiles/all_kernels_llama7b_shapes.hbm_traffic_pmc.txt.
+# scaled by what the same counter reads for isp_calibration_copy of known size: x1.9987 and x0.9986).
+# The summary of those runs is profiles/all_kernels_benchmark_shapes.hbm_traffic_pmc.txt.
 MEASURED_TRAFFIC_BYTES = {
-    "fused_add_bias_residual_rmsnorm_f16_2048x4096": 67261704,
-    "rmsnorm_f32_64x4096": 2257998,
-    "rmsnorm_f32_16384x4096": 536838689,
-    "embedding_f16_8192x4096_v32000": 133718151,
-    "qkv_bias_rope_transpose_f16_b8_s512": 146727112,
-    "swiglu_f16_prefill_8192x11008": 540815334,
-    "swiglu_f16_decode_256x11008": 16928129,
+    "fused_add_bias_residual_rmsnorm_f16_2048x4096": 67220187,
+    "rmsnorm_f32_64x4096": 2256656,
+    "rmsnorm_f32_16384x4096": 536490518,
+    "embedding_f16_8192x4096_v32000": 133616596,
+    "qkv_bias_rope_transpose_f16_b8_s512": 146643388,
+    "swiglu_f16_prefill_8192x11008": 540601380,
+    "swiglu_f16_decode_256x11008": 16921499,
+    "transpose_remove_padding_f16_b8_s512": 48954297,
+    "concat_kv_cache_f16_b8_q512_S1024": 97464471,
+    "repeat_kv_cache_f16_b8_k512_S1024": 97478542,
+    "rope_decode_f16_1x96x128": 49363,
     "calibration_copy_64MiB_traffic": 67108864,
-    "calibration_copy_512MiB_traffic": 536685713,
+    "calibration_copy_512MiB_traffic": 536471488,
 }
 
 
@@ -419,8 +423,8 @@ def main():
         "metric": "HBM GB/s & % of peak per fused kernel at LLaMA-2-7B shapes; tokens/sec",
         "value": head["GBps"], "unit": "GB/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
         "ms_per_step": head["ms_per_step_wall"], "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "f16 storage, f32 arithmetic", "data": "synthetic",
-        "config": {"workload": head["workload"], "tokens_per_s": head["tokens_per_s"],
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": head["workload"], "storage_dtype": "f16", "tokens_per_s": head["tokens_per_s"],
                    "cache": "cold: launches rotate over %d buffer sets (> 1 GiB)" % head["buffer_sets"]},
         "roofline": dict(head["roofline"], kernel=head["kernel"],
                          algorithmic_bytes_per_launch=head["algorithmic_bytes"],

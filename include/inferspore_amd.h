@@ -219,7 +219,8 @@ typedef enum isp_tuning_knob {
                                         3 = a workgroup per 4 KiB chunk of a row (default) */
     ISP_TUNE_EMBED_STORE = 5,        /* 1 = plain, 2 = non-temporal (default) */
     ISP_TUNE_QKV_STORE = 6,          /* 1 = plain, 2 = non-temporal (default) */
-    ISP_TUNE_COUNT = 7
+    ISP_TUNE_QKV_WAVES = 7,          /* waves (groups of 8 heads) per workgroup: 1, 2 or 4 (default) */
+    ISP_TUNE_COUNT = 8
 } isp_tuning_knob;
 int isp_tuning_set(int knob, int value);
 

@@ -54,8 +54,8 @@ __device__ __forceinline__ void rotate_pair(float c, float sn, float x0, float x
 // two stores), evaluates the token's (cos, sin) pairs itself (lane d evaluates pair d) and shares
 // them through a wave-private slice of LDS, so there is no workgroup barrier; waves that only carry
 // v heads skip the evaluation.  grid = (tokens, head groups of 4 waves).
-template <typename T, int HS, bool NT>
-__global__ __launch_bounds__(kBlock) void qkv_rope_wave(
+template <typename T, int HS, bool NT, int WAVES>
+__global__ __launch_bounds__(kWave * WAVES) void qkv_rope_wave(
     T* __restrict__ q, T* __restrict__ k, T* __restrict__ v, const T* __restrict__ qkv,
     const T* __restrict__ bias, const int32_t* __restrict__ padding_offset,
     const int32_t* __restrict__ history_length, int batch, int seq_len, int head_num,
@@ -65,7 +65,6 @@ __global__ __launch_bounds__(kBlock) void qkv_rope_wave(
     constexpr int G = HALF / VEC;
     static_assert(HALF % VEC == 0 && kWave % G == 0 && HALF <= kWave, "unsupported head size");
     constexpr int HEADS_PER_WAVE = kWave / G;
-    constexpr int WAVES = kBlock / kWave;
 
     // grid = (tokens, head groups): the token index runs fastest, so the workgroups in flight at any
     // time read 8 KiB slices of consecutive token rows and write into one group of 32 heads
@@ -353,15 +352,21 @@ static int qkv_rope(void* q_, void* k_, void* v_, const void* qkv_, const void* 
     dim3 grid((unsigned)token_num), block(kBlock);
     hipError_t e;
     const bool nt = tuning(ISP_TUNE_QKV_STORE) != 1;
-#define ISP_QKV_LAUNCH_1(HS, N, GRID)                                                              \
-    hipLaunchKernelGGL((qkv_rope_wave<T, HS, N>), GRID, block, 0, s, q, k, v, qkv, bias,            \
-                       padding_offset, history_length, batch, seq_len, head_num, kv_head_num,      \
-                       half_rot, tab)
+    int waves = tuning(ISP_TUNE_QKV_WAVES);
+    if (waves != 1 && waves != 2 && waves != 4) waves = 4;  // 4 measured best (8 and 12 are slower)
+#define ISP_QKV_LAUNCH_1(HS, N, W)                                                                 \
+    do {                                                                                           \
+        constexpr int HPB = (kWave / ((HS / 2) / Elem<T>::kVec)) * W;                              \
+        dim3 g2((unsigned)token_num, (unsigned)((head_num + 2 * kv_head_num + HPB - 1) / HPB));    \
+        hipLaunchKernelGGL((qkv_rope_wave<T, HS, N, W>), g2, dim3(kWave * W), 0, s, q, k, v, qkv,   \
+                           bias, padding_offset, history_length, batch, seq_len, head_num,         \
+                           kv_head_num, half_rot, tab);                                            \
+    } while (0)
 #define ISP_QKV_LAUNCH_WAVE(HS)                                                                    \
     do {                                                                                           \
-        constexpr int HPB = (kWave / ((HS / 2) / Elem<T>::kVec)) * (kBlock / kWave);               \
-        dim3 g2((unsigned)token_num, (unsigned)((head_num + 2 * kv_head_num + HPB - 1) / HPB));    \
-        if (nt) ISP_QKV_LAUNCH_1(HS, true, g2); else ISP_QKV_LAUNCH_1(HS, false, g2);              \
+        if (waves == 1) { if (nt) ISP_QKV_LAUNCH_1(HS, true, 1); else ISP_QKV_LAUNCH_1(HS, false, 1); } \
+        else if (waves == 2) { if (nt) ISP_QKV_LAUNCH_1(HS, true, 2); else ISP_QKV_LAUNCH_1(HS, false, 2); } \
+        else { if (nt) ISP_QKV_LAUNCH_1(HS, true, 4); else ISP_QKV_LAUNCH_1(HS, false, 4); }       \
     } while (0)
     const int head_groups_max = 65535 * 4;  // grid.y limit, 4 heads per workgroup at least
     if (vec_ok && head_size == 128 && head_num + 2 * kv_head_num <= head_groups_max) {

@@ -352,9 +352,9 @@ def test_knobs_do_not_change_results(isp):
             return [host(o) for o in outs]
 
         base = run_qkv()
-        for store in (1, 2):
-            say("qkv knobs %s store=%d" % (dtype.__name__, store))
-            got = _with_knobs({capi.TUNE_QKV_STORE: store}, run_qkv)
+        for store, waves in itertools.product((1, 2), (1, 2, 4)):
+            say("qkv knobs %s store=%d waves=%d" % (dtype.__name__, store, waves))
+            got = _with_knobs({capi.TUNE_QKV_STORE: store, capi.TUNE_QKV_WAVES: waves}, run_qkv)
             assert all(np.array_equal(a, b) for a, b in zip(got, base))
     # embedding
     ids, table = embedding_inputs(77, 4096, 300, np.float16, seed=43)
@@ -392,3 +392,22 @@ def test_knobs_do_not_change_results(isp):
     for store in (1, 2):
         got = _with_knobs({capi.TUNE_NORM_STORE: store}, run_norm)
         assert np.array_equal(got[0], base[0]) and np.array_equal(got[1], base[1])
+
+
+# ------------------------------------------------------------------ token counts beyond 65535 (grid limits)
+def test_large_token_counts(isp, oracle):
+    tokens = 70001
+    say("large token count: norm")
+    _check_norm(isp, oracle, np.float16, tokens, 64, True, True, seed=61)
+    say("large token count: swiglu")
+    x = swiglu_inputs(tokens, 16, np.float16, seed=62)
+    out = torch.empty((tokens, 16), dtype=torch.float16, device="cuda")
+    isp.act(dev(x), out)
+    assert_f16_close(host(out), oracle.swiglu(x), "swiglu many tokens")
+    say("large token count: embedding")
+    ids, table = embedding_inputs(tokens, 16, 100, np.float16, seed=63)
+    out = torch.empty((tokens, 16), dtype=torch.float16, device="cuda")
+    isp.input_embedding(dev(ids), out, dev(table))
+    assert np.array_equal(host(out), oracle.embedding(ids, table))
+    say("large token count: qkv")
+    _check_qkv(isp, oracle, np.float16, 1, tokens, 1, 1, 64, 64, seed=64, min_len=tokens)
