@@ -32,6 +32,18 @@ def _p(t):
     return None if t is None else t.data_ptr()
 
 
+def _same_dtype(ref, *tensors):
+    for t in tensors:
+        if t is not None and t.dtype != ref.dtype:
+            raise TypeError("inferspore_amd: operand dtype %s does not match %s" % (t.dtype, ref.dtype))
+
+
+def _int32(*tensors):
+    for t in tensors:
+        if t is not None and t.dtype != torch.int32:
+            raise TypeError("inferspore_amd: index / length tensors must be int32, got %s" % t.dtype)
+
+
 def _stream():
     return torch.cuda.current_stream().cuda_stream
 
@@ -72,6 +84,7 @@ def cal_padding_offset(padding_offset, cum_seqlens, input_lengths):
 def rmsnorm(x, gamma, eps):
     """In-place RMSNorm of x [tokens, hidden]."""
     _dev(x, gamma)
+    _same_dtype(x, gamma)
     fn = getattr(capi.lib(), "isp_rmsnorm_" + _suffix(x))
     capi.check(fn(_p(x), _p(gamma), float(eps), x.shape[0], x.shape[1], _stream()), "isp_rmsnorm")
     return x
@@ -80,6 +93,7 @@ def rmsnorm(x, gamma, eps):
 def fused_add_bias_residual_rmsnorm(residual, decoder_out, bias, gamma, eps, flags=0):
     """launchFusedAddBiasResidualRMSNorm: in place on residual (may be None) and decoder_out."""
     _dev(residual, decoder_out, bias, gamma)
+    _same_dtype(decoder_out, residual, bias, gamma)
     fn = getattr(capi.lib(), "isp_fused_add_bias_residual_rmsnorm_" + _suffix(decoder_out))
     capi.check(fn(_p(residual), _p(decoder_out), _p(bias), _p(gamma), float(eps),
                   decoder_out.shape[0], decoder_out.shape[1], int(flags), _stream()),
@@ -94,6 +108,8 @@ def add_fused_qkv_bias_transpose_and_rope(q_buf, k_buf, v_buf, qkv, qkv_bias, pa
     """launchAddFusedQKVBiasTransposeAndRoPE; shapes as the reference derives them
     (qkv_bias_and_RoPE.cu:298-304)."""
     _dev(q_buf, k_buf, v_buf, qkv, qkv_bias, padding_offset, history_length, input_length)
+    _same_dtype(qkv, q_buf, k_buf, v_buf, qkv_bias)
+    _int32(padding_offset, history_length, input_length)
     token_num, qkv_head_num, head_size = qkv.shape
     batch, head_num, seq_len = q_buf.shape[0], q_buf.shape[1], q_buf.shape[2]
     kv_head_num = (qkv_head_num - head_num) // 2
@@ -109,6 +125,7 @@ def add_fused_qkv_bias_transpose_and_rope(q_buf, k_buf, v_buf, qkv, qkv_bias, pa
 def act(input, out):
     """launchAct (SwiGLU): input [tokens, 2, inter] -> out [tokens, inter]."""
     _dev(input, out)
+    _same_dtype(input, out)
     if input.shape[1] != 2:
         raise RuntimeError("SwiGLU input must have shape [tokens, 2, inter]")
     fn = getattr(capi.lib(), "isp_swiglu_" + _suffix(input))
@@ -131,6 +148,8 @@ def rope(qkv_buf, step, head_num, rotary_embedding_dim, rotary_embedding_base):
 def transpose_out_remove_padding(qkv_buf_w_pad, padding_offset, qkv_buf_wo_pad):
     """launchTransposeOutRemovePadding: [batch, heads, seq, hs] -> [tokens, heads, hs]."""
     _dev(qkv_buf_w_pad, padding_offset, qkv_buf_wo_pad)
+    _same_dtype(qkv_buf_w_pad, qkv_buf_wo_pad)
+    _int32(padding_offset)
     batch, head_num, seq_len, head_size = qkv_buf_w_pad.shape
     token_num = qkv_buf_wo_pad.shape[0]
     fn = getattr(capi.lib(), "isp_transpose_remove_padding_" + _suffix(qkv_buf_w_pad))
@@ -142,6 +161,8 @@ def transpose_out_remove_padding(qkv_buf_w_pad, padding_offset, qkv_buf_wo_pad):
 def concat_kv_cache(k_src, v_src, layer_id, cur_query_length, history_length, k_dst, v_dst):
     """launchConcatKVCache; shapes as the reference derives them (concat_past_kv.cu:84-90)."""
     _dev(k_src, v_src, cur_query_length, history_length, k_dst, v_dst)
+    _same_dtype(k_src, v_src, k_dst, v_dst)
+    _int32(cur_query_length, history_length)
     batch, kv_head_num, max_q_len, head_size = k_src.shape
     max_seq_len = k_dst.shape[3]
     fn = getattr(capi.lib(), "isp_concat_kv_cache_" + _suffix(k_src))
@@ -154,6 +175,8 @@ def concat_kv_cache(k_src, v_src, layer_id, cur_query_length, history_length, k_
 def repeat_kv_cache(k_cache_src, v_cache_src, context_length, layer_id, k_cache_dst, v_cache_dst):
     """launchRepeatKVCache; shapes as the reference derives them (repeat_kv.cu:59-70)."""
     _dev(k_cache_src, v_cache_src, context_length, k_cache_dst, v_cache_dst)
+    _same_dtype(k_cache_src, v_cache_src, k_cache_dst, v_cache_dst)
+    _int32(context_length)
     batch = context_length.shape[0]
     kv_head_num, max_seq_len = k_cache_src.shape[2], k_cache_src.shape[3]
     head_num, max_k_len, head_size = k_cache_dst.shape[1], k_cache_dst.shape[2], k_cache_dst.shape[3]
