@@ -68,7 +68,8 @@ __global__ __launch_bounds__(kWave * WAVES) void qkv_rope_wave(
 
     // grid = (tokens, head groups): the token index runs fastest, so the workgroups in flight at any
     // time read 8 KiB slices of consecutive token rows and write into one group of 32 heads
-    // (measured: faster than token-major order and than 4-token workgroups).
+    // (measured: faster than token-major order, than 4-token workgroups, and than a layout with
+    // one vector per lane and a DPP exchange of the rotation partners).
     const int lane = threadIdx.x % kWave;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     const int token = (int)blockIdx.x;
