@@ -94,3 +94,32 @@ def test_python_layer_refuses_mismatched_dtypes():
         ops._same_dtype(torch.ones(2, dtype=torch.float16), torch.ones(2, dtype=torch.float32))
     with pytest.raises(TypeError):
         ops._int32(torch.ones(2, dtype=torch.int64))
+
+
+def test_argument_validation_of_the_neighbour_entry_points(lib):
+    from inferspore_amd import capi
+    p = ctypes.c_void_p(16)
+    rope = lib.isp_rope_decode_f16
+    assert rope(None, 0, 32, 32, 128, 5, 128, 10000.0, None) == capi.OK            # no rows: nothing to do
+    assert rope(None, 1, 32, 32, 128, 5, 128, 10000.0, None) == capi.ERR_NULL_POINTER
+    assert rope(p, 1, 32, 32, 127, 5, 126, 10000.0, None) == capi.ERR_BAD_SHAPE    # odd head size
+    assert rope(p, 1, 32, 32, 128, 5, 130, 10000.0, None) == capi.ERR_BAD_SHAPE    # rotary dim > head size
+    assert rope(p, -1, 32, 32, 128, 5, 128, 10000.0, None) == capi.ERR_BAD_SHAPE
+    tr = lib.isp_transpose_remove_padding_f32
+    assert tr(None, None, None, 2, 4, 8, 16, 0, None) == capi.OK
+    assert tr(p, None, p, 2, 4, 8, 16, 5, None) == capi.ERR_NULL_POINTER
+    assert tr(p, p, p, 0, 4, 8, 16, 5, None) == capi.ERR_BAD_SHAPE                 # tokens but no batch
+    assert tr(p, p, p, 2, -4, 8, 16, 5, None) == capi.ERR_BAD_SHAPE
+    cat = lib.isp_concat_kv_cache_f16
+    assert cat(None, None, None, None, 0, None, None, 0, 4, 8, 16, 128, None) == capi.OK
+    assert cat(p, p, p, None, 0, p, p, 2, 4, 8, 16, 128, None) == capi.ERR_NULL_POINTER
+    assert cat(p, p, p, p, -1, p, p, 2, 4, 8, 16, 128, None) == capi.ERR_BAD_SHAPE  # negative layer
+    assert cat(p, p, p, p, 0, p, p, 70000, 4, 8, 16, 128, None) == capi.ERR_UNSUPPORTED
+    rep = lib.isp_repeat_kv_cache_f32
+    assert rep(None, None, None, None, 0, None, 0, 8, 2, 16, 8, 128, None) == capi.OK
+    assert rep(p, p, p, p, 0, None, 2, 8, 2, 16, 8, 128, None) == capi.ERR_NULL_POINTER
+    assert rep(p, p, p, p, 0, p, 2, 8, 3, 16, 8, 128, None) == capi.ERR_BAD_SHAPE   # heads not a multiple of kv heads
+    assert lib.isp_calibration_copy(p, p, 24, None) == capi.ERR_BAD_SHAPE           # not a multiple of 16 bytes
+    assert lib.isp_calibration_copy(None, None, 0, None) == capi.OK
+    assert lib.isp_tuning_set(99, 1) == capi.ERR_BAD_SHAPE
+    assert lib.isp_tuning_set(capi.TUNE_NORM_STORE, 0) >= 0
