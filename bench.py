@@ -56,7 +56,7 @@ def parse():
     ap.add_argument("--only", default=None, help="run a single workload by name")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--warm", action="store_true", help="also report cache-warm (no rotation) rates")
-    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline leg")
+    ap.add_argument("--cpu-seconds", type=float, default=20.0, help="budget of the CPU baseline leg")
     return ap.parse_args()
 
 
@@ -114,7 +114,16 @@ def make_workloads(torch, lib, stream_handle, rotate):
         bias = (0.02 * torch.randn(hidden, device=dev)).to(tdtype) if fused else None
         gamma = (0.5 + torch.rand(hidden, device=dev)).to(tdtype)
         w.keep = (outs, ress, bias, gamma)
-        w.kernel = "isp::fused_norm_rows<%s, ...>" % ("__half" if es == 2 else "float")
+        # the instantiation the launch heuristic picks for this shape (vectors per lane, waves per row)
+        nvec = hidden // (16 // es)
+        wpr = 1
+        while wpr < 16 and -(-nvec // (64 * wpr)) > 2:
+            wpr *= 2
+        while wpr < 16 and -(-nvec // (64 * wpr)) > 1 and tokens * wpr < 4096:
+            wpr *= 2
+        nv = -(-nvec // (64 * wpr))
+        nv = 1 if nv <= 1 else 2 if nv <= 2 else 4 if nv <= 4 else 8
+        w.kernel = "isp::fused_norm_rows<%s, %d, %d, true>" % ("__half" if es == 2 else "float", nv, wpr)
         if fused:
             fn = getattr(lib, "isp_fused_add_bias_residual_rmsnorm_" + sfx)
             w.bind(fn, [(ress[j].data_ptr(), outs[j].data_ptr(), bias.data_ptr(), gamma.data_ptr(), 1e-5, tokens,
@@ -378,48 +387,147 @@ def context_layer_record(torch, steps, warmup, stream):
             "note": "library kernels via the C ABI; GEMMs and attention are torch library calls"}
 
 
+def decode_sequence_record(torch, stream):
+    """The launch-bound side: one decode step's worth of this library's kernels (batch 16: fused norm,
+    decode RoPE, KV append, KV broadcast, SwiGLU, RMSNorm) issued eagerly and replayed from a captured
+    HIP graph -- the entry points record only kernel nodes, so a caller can amortise launch latency."""
+    from inferspore_amd import ops
+    batch, kvn, hn, hs, max_seq, inter = 16, 32, 32, 128, 256, 11008
+    with torch.cuda.stream(stream):
+        h = lambda *sh: torch.randn(sh, device="cuda").half()
+        hidden, residual, gamma = h(batch, 4096), h(batch, 4096), h(4096)
+        qkv = h(1, 96, 128)
+        k_new, v_new = h(batch, kvn, 1, hs), h(batch, kvn, 1, hs)
+        ones = torch.ones(batch, dtype=torch.int32, device="cuda")
+        hist, ctx = ones * 100, ones * 101
+        k_cache, v_cache = h(1, batch, kvn, max_seq, hs), h(1, batch, kvn, max_seq, hs)
+        k_rep = torch.zeros((batch, hn, 101, hs), dtype=torch.float16, device="cuda")
+        v_rep = torch.zeros_like(k_rep)
+        gate_up, act_out = h(batch, 2, inter), torch.zeros((batch, inter), dtype=torch.float16, device="cuda")
+
+        def step():
+            ops.fused_add_bias_residual_rmsnorm(residual, hidden, None, gamma, 1e-5)
+            ops.rope(qkv, 101, 32, 128, 10000.0)
+            ops.concat_kv_cache(k_new, v_new, 0, ones, hist, k_cache, v_cache)
+            ops.repeat_kv_cache(k_cache, v_cache, ctx, 0, k_rep, v_rep)
+            ops.act(gate_up, act_out)
+            ops.rmsnorm(hidden, gamma, 1e-5)
+
+        def timed(fn, n):
+            for _ in range(5):
+                fn()
+            stream.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(stream)
+            for _ in range(n):
+                fn()
+            e1.record(stream)
+            stream.synchronize()
+            return e0.elapsed_time(e1) * 1e3 / n
+
+        eager_us = timed(step, 200)
+        graph = torch.cuda.CUDAGraph()
+        graph.capture_begin()
+        step()
+        graph.capture_end()
+        stream.synchronize()
+        graph_us = timed(graph.replay, 200)
+    return {"workload": "decode_step_sequence_b16 (6 kernels)", "eager_us_per_step": eager_us,
+            "graph_replay_us_per_step": graph_us, "kernels_per_step": 6}
+
+
 # --------------------------------------------------------------------------- CPU baseline
 
 def cpu_baseline(budget_s):
-    """Times the C oracle (port of the reference's CPU functions) on the headline workload shape."""
+    """Times the C oracle (a port of the reference's CPU test functions) on the host cores, per kernel,
+    on bounded samples of the benchmark workloads: single thread (as the reference's loops are written)
+    and OpenMP over token rows.  The headline entry is the fused norm at its full size."""
     import numpy as np
     sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
     from oracle import load
     o = load()
-    tokens, hidden = 2048, 4096
+    L = o.lib
     r = np.random.default_rng(0)
-    out = r.standard_normal((tokens, hidden)).astype(np.float16)
-    res = r.standard_normal((tokens, hidden)).astype(np.float16)
-    bias = (0.02 * r.standard_normal(hidden)).astype(np.float16)
-    gamma = r.uniform(0.5, 1.5, hidden).astype(np.float16)
-    nbytes = 4 * tokens * hidden * 2 + 2 * hidden * 2
+    f16 = np.float16
 
-    def run(threads, budget):
+    def normal(*shape, scale=1.0, dtype=f16):
+        return (scale * r.standard_normal(shape, dtype=np.float32)).astype(dtype)
+
+    samples = []   # (workload, description, tokens, algorithmic bytes, callable, fresh-inputs callable or None)
+
+    tokens, hidden = 2048, 4096
+    out, res = normal(tokens, hidden), normal(tokens, hidden)
+    bias, gamma = normal(hidden, scale=0.02), r.uniform(0.5, 1.5, hidden).astype(f16)
+    wa, wb = out.copy(), res.copy()
+
+    def norm_reset():
+        wa[...] = out
+        wb[...] = res
+    samples.append(("fused_add_bias_residual_rmsnorm_f16_2048x4096", "full workload", tokens,
+                    4 * tokens * hidden * 2 + 2 * hidden * 2,
+                    lambda: L.isp_oracle_fused_norm_f16(wb.ctypes.data, wa.ctypes.data, bias.ctypes.data,
+                                                        gamma.ctypes.data, 1e-5, tokens, hidden, 0), norm_reset))
+    x32 = normal(64, hidden, dtype=np.float32)
+    g32 = r.uniform(0.5, 1.5, hidden).astype(np.float32)
+    w32 = x32.copy()
+    samples.append(("rmsnorm_f32_64x4096", "full workload", 64, 2 * 64 * hidden * 4 + hidden * 4,
+                    lambda: L.isp_oracle_fused_norm_f32(None, w32.ctypes.data, None, g32.ctypes.data, 1e-5, 64,
+                                                        hidden, 0), lambda: w32.__setitem__(Ellipsis, x32)))
+    et, vocab = 8192, 32000
+    table = np.full((vocab, hidden), 0.01, f16)
+    ids = r.integers(0, vocab, et, dtype=np.int32)
+    eo = np.empty((et, hidden), f16)
+    samples.append(("embedding_f16_8192x4096_v32000", "full workload", et, 2 * et * hidden * 2 + et * 4,
+                    lambda: L.isp_oracle_embedding(ids.ctypes.data, eo.ctypes.data, table.ctypes.data, et, hidden, 2),
+                    None))
+    qt, heads, hs, seq = 256, 96, 128, 512
+    qkv, qb = normal(qt, heads, hs), normal(heads * hs, scale=0.02)
+    qo = [np.zeros((1, 32, seq, hs), f16) for _ in range(3)]
+    po, hist, ilen = np.zeros(qt, np.int32), np.zeros(1, np.int32), np.full(1, qt, np.int32)
+    samples.append(("qkv_bias_rope_transpose_f16_b8_s512", "one sequence of 256 tokens (of 2977)", qt,
+                    qt * (2 * heads * hs * 2 + 4) + heads * hs * 2,
+                    lambda: L.isp_oracle_qkv_rope_f16(qo[0].ctypes.data, qo[1].ctypes.data, qo[2].ctypes.data,
+                                                      qkv.ctypes.data, qb.ctypes.data, po.ctypes.data,
+                                                      hist.ctypes.data, ilen.ctypes.data, 1, seq, qt, 32, 32, hs,
+                                                      128, 10000.0), None))
+    st, inter = 256, 11008
+    sx, so = normal(st, 2, inter), np.empty((st, inter), f16)
+    samples.append(("swiglu_f16_decode_256x11008", "full workload (= 256 of the 8192 prefill tokens)", st,
+                    st * 3 * inter * 2,
+                    lambda: L.isp_oracle_swiglu_f16(sx.ctypes.data, so.ctypes.data, st, inter), None))
+
+    def timed(fn, reset, threads, budget):
         o.set_threads(threads)
-        lib = o.lib
         times = []
         t_end = time.perf_counter() + budget
-        a, b = out.copy(), res.copy()
-        while len(times) < 3 or (time.perf_counter() < t_end and len(times) < 50):
-            a[...] = out
-            b[...] = res
+        while len(times) < 2 or (time.perf_counter() < t_end and len(times) < 30):
+            if reset:
+                reset()
             t0 = time.perf_counter()
-            lib.isp_oracle_fused_norm_f16(b.ctypes.data, a.ctypes.data, bias.ctypes.data, gamma.ctypes.data,
-                                          1e-5, tokens, hidden, 0)
+            fn()
             times.append(time.perf_counter() - t0)
         o.set_threads(1)
         times.sort()
         return times[len(times) // 2], len(times)
 
-    t1, n1 = run(1, budget_s * 0.6)
     cores = min(16, o.max_threads())
-    tn, nn = run(cores, budget_s * 0.4)
+    per = budget_s / (2.0 * len(samples))
+    records = []
+    for name, what, toks, nbytes, fn, reset in samples:
+        t1, n1 = timed(fn, reset, 1, per * 1.4)
+        tn, nn = timed(fn, reset, cores, per * 0.6)
+        records.append({"workload": name, "sample": what, "kind": "port",
+                        "one_thread": {"GBps": nbytes / t1 / 1e9, "tokens_per_s": toks / t1, "cores": 1, "runs": n1},
+                        "openmp": {"GBps": nbytes / tn / 1e9, "tokens_per_s": toks / tn, "cores": cores, "runs": nn}})
+    head = records[0]
     return {
-        "value": nbytes / t1 / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
-        "sample": "full workload (2048x4096 fp16 fused add-bias+residual+RMSNorm), median of %d runs" % n1,
-        "tokens_per_s": tokens / t1,
-        "openmp": {"value": nbytes / tn / 1e9, "unit": "GB/s", "cores": cores, "tokens_per_s": tokens / tn,
-                   "runs": nn},
+        "value": head["one_thread"]["GBps"], "unit": "GB/s", "cores": 1, "kind": "port",
+        "sample": "full workload (2048x4096 fp16 fused add-bias+residual+RMSNorm), median of %d runs"
+                  % head["one_thread"]["runs"],
+        "tokens_per_s": head["one_thread"]["tokens_per_s"],
+        "openmp": {"value": head["openmp"]["GBps"], "unit": "GB/s", "cores": cores,
+                   "tokens_per_s": head["openmp"]["tokens_per_s"]},
+        "per_kernel": records,
     }
 
 
@@ -482,6 +590,7 @@ def main():
         layer["library_kernels_ms_estimate"] = est
         layer["library_kernels_share"] = est / layer["ms_per_layer"]
         line["context_layer"] = layer
+        line["decode_sequence"] = decode_sequence_record(torch, stream)
     if a.warm:
         line["warm_cache"] = {r["workload"]: {"GBps": r["GBps"], "ms_per_launch_events": r["ms_per_launch_events"]}
                               for r in run_all(False)}
