@@ -17,11 +17,39 @@
 
 namespace isp {
 
+// Vectors per head row: almost always a power of two (16 for 128 fp16 elements), so the row / column
+// split of a flat vector index is a shift and a mask; any other width takes the division.
+struct SegSplit {
+    unsigned seg_vec;
+    int shift;  // log2(seg_vec) or -1
+    __device__ __forceinline__ void split(unsigned vi, unsigned& row, unsigned& col) const {
+        if (shift >= 0) {
+            row = vi >> shift;
+            col = vi & (seg_vec - 1u);
+        } else {
+            row = vi / seg_vec;
+            col = vi - row * seg_vec;
+        }
+    }
+};
+
+static SegSplit make_split(unsigned seg_vec) {
+    SegSplit sp;
+    sp.seg_vec = seg_vec;
+    sp.shift = -1;
+    if (seg_vec != 0 && (seg_vec & (seg_vec - 1u)) == 0) {
+        sp.shift = 0;
+        while ((1u << sp.shift) < seg_vec) sp.shift++;
+    }
+    return sp;
+}
+
 // dst[token, h, :] = src[b, h, s, :],  token + padding_offset[token] = b * seq_len + s.
 // grid = tokens * chunks, a chunk being 256 vectors of the token's heads*seg_vec vectors
 __global__ __launch_bounds__(kBlock) void transpose_remove_padding_vec(
     const char* __restrict__ src, const int32_t* __restrict__ padding_offset, char* __restrict__ dst,
-    int batch, int head_num, int seq_len, unsigned seg_vec, unsigned chunks) {
+    int batch, int head_num, int seq_len, SegSplit sp, unsigned chunks) {
+    const unsigned seg_vec = sp.seg_vec;
     const unsigned token = blockIdx.x / chunks;
     const unsigned vi = (blockIdx.x % chunks) * kBlock + threadIdx.x;  // vector index inside the token's row
     const unsigned row_vec = (unsigned)head_num * seg_vec;
@@ -29,7 +57,8 @@ __global__ __launch_bounds__(kBlock) void transpose_remove_padding_vec(
     const long long p = (long long)token + (long long)padding_offset[token];
     if (p < 0 || p >= (long long)batch * seq_len) return;
     const unsigned b = (unsigned)(p / seq_len), s = (unsigned)(p % seq_len);
-    const unsigned h = vi / seg_vec, c = vi % seg_vec;
+    unsigned h, c;
+    sp.split(vi, h, c);
     const size_t from = ((((size_t)b * head_num + h) * seq_len + s) * seg_vec + c) * 16u;
     store16_stream(dst + ((size_t)token * row_vec + vi) * 16u, load16_stream(src + from));
 }
@@ -54,14 +83,16 @@ __global__ __launch_bounds__(kBlock) void concat_kv_vec(
     const char* __restrict__ k_src, const char* __restrict__ v_src, char* __restrict__ k_cache,
     char* __restrict__ v_cache, const int32_t* __restrict__ cur_query_length,
     const int32_t* __restrict__ history_length, int kv_head_num, int max_q_len, int max_seq_len,
-    unsigned seg_vec) {
+    SegSplit sp) {
+    const unsigned seg_vec = sp.seg_vec;
     const char* src = blockIdx.z == 0 ? k_src : v_src;
     char* cache = blockIdx.z == 0 ? k_cache : v_cache;
     const unsigned bh = blockIdx.y;
     const unsigned b = bh / kv_head_num;
     const unsigned vi = blockIdx.x * kBlock + threadIdx.x;
     if (vi >= (unsigned)max_q_len * seg_vec) return;
-    const unsigned t = vi / seg_vec, c = vi % seg_vec;
+    unsigned t, c;
+    sp.split(vi, t, c);
     const int cur = cur_query_length[b];
     const long long row = (long long)history_length[b] + t;
     if ((int)t >= cur || row < 0 || row >= max_seq_len) return;
@@ -88,14 +119,16 @@ __global__ __launch_bounds__(kBlock) void concat_kv_bytes(
 __global__ __launch_bounds__(kBlock) void repeat_kv_vec(
     const char* __restrict__ k_cache, const char* __restrict__ v_cache, char* __restrict__ k_dst,
     char* __restrict__ v_dst, const int32_t* __restrict__ context_length, int head_num,
-    int kv_head_num, int max_seq_len, int max_k_len, unsigned seg_vec) {
+    int kv_head_num, int max_seq_len, int max_k_len, SegSplit sp) {
+    const unsigned seg_vec = sp.seg_vec;
     const char* cache = blockIdx.z == 0 ? k_cache : v_cache;
     char* dst = blockIdx.z == 0 ? k_dst : v_dst;
     const unsigned bh = blockIdx.y;
     const unsigned b = bh / head_num, h = bh % head_num;
     const unsigned vi = blockIdx.x * kBlock + threadIdx.x;
     if (vi >= (unsigned)max_k_len * seg_vec) return;
-    const unsigned s = vi / seg_vec;
+    unsigned s, c;
+    sp.split(vi, s, c);
     if ((int)s >= context_length[b] || (int)s >= max_seq_len) return;
     const unsigned kvh = h / (unsigned)(head_num / kv_head_num);
     store16_stream(dst + ((size_t)bh * max_k_len * seg_vec + vi) * 16u,
@@ -134,7 +167,7 @@ static int transpose_remove_padding(const void* src, const int32_t* padding_offs
         dim3 grid((unsigned)(chunks * (size_t)token_num));
         hipLaunchKernelGGL(transpose_remove_padding_vec, grid, dim3(kBlock), 0, s,
                            static_cast<const char*>(src), padding_offset, static_cast<char*>(dst),
-                           batch, head_num, seq_len, seg_vec, (unsigned)chunks);
+                           batch, head_num, seq_len, make_split(seg_vec), (unsigned)chunks);
     } else {
         hipLaunchKernelGGL(transpose_remove_padding_bytes, dim3((unsigned)token_num), dim3(kBlock), 0,
                            s, static_cast<const char*>(src), padding_offset, static_cast<char*>(dst),
@@ -170,7 +203,7 @@ static int concat_kv(const void* k_src, const void* v_src, void* k_cache, void* 
         if (row_vec > 0xffffffffull) return ISP_ERR_UNSUPPORTED;
         dim3 grid((unsigned)((row_vec + kBlock - 1) / kBlock), (unsigned)(batch * kv_head_num), 2);
         hipLaunchKernelGGL(concat_kv_vec, grid, dim3(kBlock), 0, s, ks, vs, kc, vc, cur_query_length,
-                           history_length, kv_head_num, max_q_len, max_seq_len, seg_vec);
+                           history_length, kv_head_num, max_q_len, max_seq_len, make_split(seg_vec));
     } else {
         dim3 grid((unsigned)max_q_len, (unsigned)(batch * kv_head_num), 2);
         hipLaunchKernelGGL(concat_kv_bytes, grid, dim3(kBlock), 0, s, ks, vs, kc, vc, cur_query_length,
@@ -205,7 +238,7 @@ static int repeat_kv(const void* k_cache, const void* v_cache, void* k_dst, void
         if (row_vec > 0xffffffffull) return ISP_ERR_UNSUPPORTED;
         dim3 grid((unsigned)((row_vec + kBlock - 1) / kBlock), (unsigned)(batch * head_num), 2);
         hipLaunchKernelGGL(repeat_kv_vec, grid, dim3(kBlock), 0, s, kc, vc, kd, vd, context_length,
-                           head_num, kv_head_num, max_seq_len, max_k_len, seg_vec);
+                           head_num, kv_head_num, max_seq_len, max_k_len, make_split(seg_vec));
     } else {
         dim3 grid((unsigned)max_k_len, (unsigned)(batch * head_num), 2);
         hipLaunchKernelGGL(repeat_kv_bytes, grid, dim3(kBlock), 0, s, kc, vc, kd, vd, context_length,
