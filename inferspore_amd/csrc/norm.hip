@@ -81,6 +81,14 @@ __global__ __launch_bounds__(norm_block(WPR)) void fused_norm_rows(T* __restrict
         }
     }
 
+    // gamma is requested once this lane's part of the row has arrived and been summed: the L2 round
+    // trip then overlaps the reduction and the barrier instead of following them
+    vec16 vg[NV];
+#pragma unroll
+    for (int j = 0; j < NV; j++) {
+        if (ok[j]) vg[j] = load16(gamma + (size_t)(lane + j * ROW_THREADS) * VEC);
+    }
+
     float total = wave_sum(acc);
     if (WPR > 1) {
         __shared__ float partial[BLOCK / kWave];
@@ -98,7 +106,7 @@ __global__ __launch_bounds__(norm_block(WPR)) void fused_norm_rows(T* __restrict
         if (ok[j]) {
             const int vi = lane + j * ROW_THREADS;
             float g[VEC];
-            Elem<T>::unpack(load16(gamma + (size_t)vi * VEC), g);
+            Elem<T>::unpack(vg[j], g);
             float y[VEC];
 #pragma unroll
             for (int e = 0; e < VEC; e++) y[e] = g[e] * x[j][e] * inv;
