@@ -50,9 +50,10 @@ __global__ __launch_bounds__(norm_block(WPR)) void fused_norm_rows(T* __restrict
         }
     }
 
-    // bias and gamma are deliberately loaded where they are used, not up front with the rows: issued at
-    // kernel start, every workgroup hits the same few L2 lines at once and the streaming loads queue up
-    // behind them (measured: 13.3 us instead of 11.7 us at 2048 x 4096 fp16).
+    // bias and gamma are deliberately not requested up front with the rows: issued at kernel start,
+    // every workgroup hits the same few L2 lines at once and the streaming loads queue up behind them
+    // (measured: 13.3 us instead of 11.7 us at 2048 x 4096 fp16).  bias is loaded where it is used,
+    // gamma once the row has been summed (below).
     float x[NV][VEC];
     float acc = 0.0f;
 #pragma unroll
