@@ -74,7 +74,10 @@ def build(verbose=False, jobs=8, cpp_tests=True):
         _run([hipcc()] + HIPCC_FLAGS + ["-x", "hip", "-shared", launch_src, "-o", LIB_LAUNCH,
                                         "-L" + LIBDIR, "-linferspore_amd", "-Wl,-rpath,$ORIGIN"])
         if cpp_tests and os.path.isdir(CPPTESTS):
+            # the test programs (not the libraries) link the CPU oracle they check against
             oracle_dir = os.path.join(ROOT, "oracle")
+            if not os.path.exists(os.path.join(oracle_dir, "libisp_oracle.so")):
+                _run(["make", "-C", oracle_dir])
             srcs = sorted(f for f in os.listdir(CPPTESTS) if f.endswith(".cc"))
 
             def one(f):
@@ -83,7 +86,8 @@ def build(verbose=False, jobs=8, cpp_tests=True):
                     "-x", "hip", os.path.join(CPPTESTS, f), "-o", exe, "-I" + oracle_dir,
                     "-L" + LIBDIR, "-linferspore_launch", "-linferspore_amd",
                     "-L" + oracle_dir, "-lisp_oracle",
-                    "-Wl,-rpath," + LIBDIR, "-Wl,-rpath," + oracle_dir])
+                    # relative to build/bin, so the tree can be moved or mounted elsewhere
+                    "-Wl,-rpath,$ORIGIN/../../inferspore_amd/lib", "-Wl,-rpath,$ORIGIN/../../oracle"])
 
             with cf.ThreadPoolExecutor(max_workers=jobs) as ex:
                 list(ex.map(one, srcs))
