@@ -96,6 +96,7 @@ int isp_rmsnorm_f16(void* x, const void* gamma, float eps, int tokens, int hidde
  *                                           literal store order, .cu:62-67)
  *   decoder_out := gamma * x * rsqrt(mean(x^2) + eps)
  *   residual, decoder_out [tokens, hidden]; bias, gamma [hidden]; residual and bias may be NULL.
+ *   residual and decoder_out must be distinct buffers (each is read and written once).
  */
 int isp_fused_add_bias_residual_rmsnorm_f32(void* residual, void* decoder_out, const void* bias,
                                             const void* gamma, float eps, int tokens, int hidden,
@@ -116,7 +117,8 @@ int isp_fused_add_bias_residual_rmsnorm_f16(void* residual, void* decoder_out, c
  * s = p % seq_len) and is rotated at timestep history_length[b] + s.  Padded positions are not
  * written.  A token whose p falls outside [0, batch * seq_len) is skipped (the reference would
  * write out of bounds).  `max_position_embeddings` and `use_dynamic_ntk` are accepted and ignored,
- * as in the reference (.cu:126-127).
+ * as in the reference (.cu:126-127).  The outputs must not overlap the input.
+ * head_size must be even, rotary_embedding_dim even and <= min(head_size, 256).
  */
 int isp_qkv_bias_rope_transpose_f32(void* q, void* k, void* v, const void* qkv, const void* bias,
                                     const int32_t* padding_offset, const int32_t* history_length,

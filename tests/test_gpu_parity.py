@@ -313,6 +313,12 @@ def test_qkv_rope_large_positions_fp32(isp, oracle):
     _check_qkv(isp, oracle, np.float32, 2, 64, 4, 4, 128, 128, seed=8, history=[4000, 2500])
 
 
+def test_qkv_rope_very_large_positions(isp, oracle):
+    # timesteps beyond 100 000: angles of 1e5 rad need the full-range argument reduction of sincosf
+    for dtype in (np.float32, np.float16):
+        _check_qkv(isp, oracle, dtype, 2, 32, 4, 4, 128, 128, seed=12, history=[131000, 99999])
+
+
 def test_qkv_rope_skips_tokens_that_fall_outside(isp):
     hn, hs, seq, batch = 2, 128, 4, 1
     qkv = torch.ones((3, 3 * hn, hs), dtype=torch.float16, device="cuda")
