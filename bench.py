@@ -563,6 +563,17 @@ def main():
             torch.cuda.empty_cache()
         return out
 
+    # bring the device out of its idle clocks before the first timed region (the headline workload is
+    # measured first): ~50 ms of streaming copies, untimed
+    with torch.cuda.stream(stream):
+        a_buf = torch.empty(64 << 20, dtype=torch.uint8, device="cuda")
+        b_buf = torch.empty(64 << 20, dtype=torch.uint8, device="cuda")
+        for _ in range(2000):
+            lib.isp_calibration_copy(b_buf.data_ptr(), a_buf.data_ptr(), 64 << 20, handle)
+        stream.synchronize()
+        del a_buf, b_buf
+    torch.cuda.empty_cache()
+
     results = run_all(True)
     head = results[0]
     line = {

@@ -214,13 +214,14 @@ int isp_calibration_copy(void* dst, const void* src, size_t bytes, isp_stream_t 
 
 typedef enum isp_tuning_knob {
     ISP_TUNE_NORM_WAVES_PER_ROW = 0, /* 1, 2, 4, 8 or 16 waves cooperate on one token row */
-    ISP_TUNE_NORM_STORE = 1,         /* output stores: 1 = plain, 2 = non-temporal (default) */
+    ISP_TUNE_NORM_STORE = 1,         /* output stores: 1 = plain, 2 = non-temporal (default),
+                                        3 = non-temporal write-through */
     ISP_TUNE_SWIGLU_UNROLL = 2,      /* 1 (default), 2 or 4 vector pairs in flight per lane */
-    ISP_TUNE_SWIGLU_STORE = 3,       /* 1 = plain, 2 = non-temporal (default) */
+    ISP_TUNE_SWIGLU_STORE = 3,       /* 1 = plain, 2 = non-temporal (default), 3 = write-through */
     ISP_TUNE_EMBED_VARIANT = 4,      /* 1 = a wave per row, 2 = a workgroup per row,
                                         3 = a workgroup per 4 KiB chunk of a row (default) */
-    ISP_TUNE_EMBED_STORE = 5,        /* 1 = plain, 2 = non-temporal (default) */
-    ISP_TUNE_QKV_STORE = 6,          /* 1 = plain, 2 = non-temporal (default) */
+    ISP_TUNE_EMBED_STORE = 5,        /* 1 = plain, 2 = non-temporal, 3 = write-through (default) */
+    ISP_TUNE_QKV_STORE = 6,          /* 1 = plain, 2 = non-temporal, 3 = write-through (default) */
     ISP_TUNE_QKV_WAVES = 7,          /* waves (groups of 8 heads) per workgroup: 1, 2 or 4 (default) */
     ISP_TUNE_COUNT = 8
 } isp_tuning_knob;

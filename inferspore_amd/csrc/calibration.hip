@@ -19,7 +19,7 @@ __global__ __launch_bounds__(kBlock) void copy_vec(char* __restrict__ dst,
 #pragma unroll
     for (int k = 0; k < UNROLL; k++) {
         const size_t v = first + (size_t)k * kBlock;
-        if (v < nvec) store16_stream(dst + v * 16, buf[k]);
+        if (v < nvec) store16_through(dst + v * 16, buf[k]);
     }
 }
 

@@ -12,7 +12,7 @@ namespace isp {
 
 // ROW_THREADS lanes (a wave, or the whole workgroup) share one row; each lane moves UNROLL vectors
 // per trip, strided by ROW_THREADS.
-template <int ROW_THREADS, int UNROLL, bool NT>
+template <int ROW_THREADS, int UNROLL, int ST>
 __global__ __launch_bounds__(kBlock) void gather_rows_vec(const int32_t* __restrict__ ids,
                                                           char* __restrict__ out,
                                                           const char* __restrict__ table, int tokens,
@@ -43,13 +43,13 @@ __global__ __launch_bounds__(kBlock) void gather_rows_vec(const int32_t* __restr
 #pragma unroll
         for (int k = 0; k < UNROLL; k++) {
             const unsigned v = v0 + k * ROW_THREADS;
-            if (v < row_vec) store16_sel<NT>(dst + (size_t)v * 16u, buf[k]);
+            if (v < row_vec) store16_sel<ST>(dst + (size_t)v * 16u, buf[k]);
         }
     }
 }
 
 // One 16-byte vector per lane: a workgroup moves one 4 KiB chunk of one row.
-template <bool NT>
+template <int ST>
 __global__ __launch_bounds__(kBlock) void gather_chunks_vec(const int32_t* __restrict__ ids,
                                                             char* __restrict__ out,
                                                             const char* __restrict__ table,
@@ -64,7 +64,7 @@ __global__ __launch_bounds__(kBlock) void gather_chunks_vec(const int32_t* __res
     vec16 buf;
     if (in_range) buf = load16_stream(table + (size_t)id * row_bytes + (size_t)v * 16u);
     else buf.w[0] = buf.w[1] = buf.w[2] = buf.w[3] = 0u;
-    store16_sel<NT>(out + (size_t)row * row_bytes + (size_t)v * 16u, buf);
+    store16_sel<ST>(out + (size_t)row * row_bytes + (size_t)v * 16u, buf);
 }
 
 // Rows that are not a whole number of aligned 16-byte vectors: one workgroup per row, byte copies.
@@ -79,6 +79,23 @@ __global__ __launch_bounds__(kBlock) void gather_rows_bytes(const int32_t* ids, 
     for (size_t i = threadIdx.x; i < row_bytes; i += kBlock) dst[i] = in_range ? src[i] : (char)0;
 }
 
+template <int ST>
+static void launch_gather(int variant, const int32_t* ids, char* o, const char* t, int tokens,
+                          unsigned row_vec, int vocab, hipStream_t s) {
+    const dim3 block(kBlock);
+    const size_t chunks = (row_vec + kBlock - 1) / kBlock;
+    if (variant == 1) {  // one wave per row
+        hipLaunchKernelGGL((gather_rows_vec<kWave, 4, ST>), dim3((unsigned)((tokens + 3) / 4)), block, 0, s,
+                           ids, o, t, tokens, row_vec, vocab);
+    } else if (variant == 2 || (size_t)tokens * chunks > 0x7fffffffull) {  // one workgroup per row
+        hipLaunchKernelGGL((gather_rows_vec<kBlock, 2, ST>), dim3((unsigned)tokens), block, 0, s, ids, o, t,
+                           tokens, row_vec, vocab);
+    } else {  // one 4 KiB chunk of a row per workgroup, one vector per lane
+        hipLaunchKernelGGL((gather_chunks_vec<ST>), dim3((unsigned)((size_t)tokens * chunks)), block, 0, s,
+                           ids, o, t, (unsigned)chunks, row_vec, vocab);
+    }
+}
+
 static int embedding(const int32_t* ids, void* out, const void* table, int tokens, int hidden,
                      int vocab, int elem_size, hipStream_t s) {
     if (tokens < 0 || hidden < 0 || vocab < 0) return ISP_ERR_BAD_SHAPE;
@@ -89,25 +106,14 @@ static int embedding(const int32_t* ids, void* out, const void* table, int token
     const size_t row_bytes = (size_t)hidden * (size_t)elem_size;
     hipError_t e;
     if (row_bytes % 16 == 0 && aligned16(out) && aligned16(table)) {
-        const bool nt = tuning(ISP_TUNE_EMBED_STORE) != 1;
+        const int kind = store_kind(tuning(ISP_TUNE_EMBED_STORE), kStoreThrough);
         const unsigned row_vec = (unsigned)(row_bytes / 16);
         char* o = static_cast<char*>(out);
         const char* t = static_cast<const char*>(table);
         const int variant = tuning(ISP_TUNE_EMBED_VARIANT);
-        if (variant == 1) {  // one wave per row
-            dim3 grid((unsigned)((tokens + 3) / 4)), block(kBlock);
-            if (nt) hipLaunchKernelGGL((gather_rows_vec<kWave, 4, true>), grid, block, 0, s, ids, o, t, tokens, row_vec, vocab);
-            else hipLaunchKernelGGL((gather_rows_vec<kWave, 4, false>), grid, block, 0, s, ids, o, t, tokens, row_vec, vocab);
-        } else if (variant == 2 || (size_t)tokens * ((row_vec + kBlock - 1) / kBlock) > 0x7fffffffull) {
-            dim3 grid((unsigned)tokens), block(kBlock);  // one workgroup per row
-            if (nt) hipLaunchKernelGGL((gather_rows_vec<kBlock, 2, true>), grid, block, 0, s, ids, o, t, tokens, row_vec, vocab);
-            else hipLaunchKernelGGL((gather_rows_vec<kBlock, 2, false>), grid, block, 0, s, ids, o, t, tokens, row_vec, vocab);
-        } else {  // one 4 KiB chunk of a row per workgroup, one vector per lane
-            const unsigned chunks = (row_vec + kBlock - 1) / kBlock;
-            dim3 grid((unsigned)tokens * chunks), block(kBlock);
-            if (nt) hipLaunchKernelGGL((gather_chunks_vec<true>), grid, block, 0, s, ids, o, t, chunks, row_vec, vocab);
-            else hipLaunchKernelGGL((gather_chunks_vec<false>), grid, block, 0, s, ids, o, t, chunks, row_vec, vocab);
-        }
+        if (kind == kStoreThrough) launch_gather<kStoreThrough>(variant, ids, o, t, tokens, row_vec, vocab, s);
+        else if (kind == kStoreStream) launch_gather<kStoreStream>(variant, ids, o, t, tokens, row_vec, vocab, s);
+        else launch_gather<kStorePlain>(variant, ids, o, t, tokens, row_vec, vocab, s);
         e = hipGetLastError();
     } else {
         hipLaunchKernelGGL(gather_rows_bytes, dim3((unsigned)tokens), dim3(kBlock), 0, s, ids,

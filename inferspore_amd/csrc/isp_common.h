@@ -55,10 +55,35 @@ __device__ __forceinline__ void store16_stream(void* p, const vec16& v) {
     u4 t = {v.w[0], v.w[1], v.w[2], v.w[3]};
     __builtin_nontemporal_store(t, reinterpret_cast<u4*>(p));
 }
+// Non-temporal and written through the XCD's L2 (agent scope, "sc1 nt") instead of being left there
+// dirty for a later write-back.  On a streaming copy: 5.0 TB/s with plain stores, 5.27 with "nt",
+// 5.57 with "sc1 nt" (64 MiB of traffic); it helps the kernels that write to fresh memory (gather,
+// QKV scatter, cache movers) and hurts the in-place norm and SwiGLU by 2 %, so it is a per-kernel
+// choice.  The compiler has no builtin for this combination on a 16-byte vector, hence the
+// one-instruction asm.  It is a vector-memory store like any other; the only thing the compiler does
+// not see is its entry in the vector-memory counter, which can only make the waits it computes for
+// later loads longer, never shorter (loads complete in order among themselves).
+__device__ __forceinline__ void store16_through(void* p, const vec16& v) {
+    typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+    u4 t = {v.w[0], v.w[1], v.w[2], v.w[3]};
+    asm volatile("global_store_dwordx4 %0, %1, off sc1 nt" : : "v"(p), "v"(t) : "memory");
+}
 
-template <bool NT>
+// Store kinds selectable per kernel instantiation.
+constexpr int kStorePlain = 0, kStoreStream = 1, kStoreThrough = 2;
+
+template <int ST>
 __device__ __forceinline__ void store16_sel(void* p, const vec16& v) {
-    if (NT) store16_stream(p, v); else store16(p, v);
+    if (ST == kStoreThrough) store16_through(p, v);
+    else if (ST == kStoreStream) store16_stream(p, v);
+    else store16(p, v);
+}
+
+// Maps a store knob (0 = the kernel's own default, 1 = plain, 2 = non-temporal, 3 = non-temporal
+// write-through) to a store kind.
+inline int store_kind(int knob_value, int default_kind) {
+    return knob_value == 1 ? kStorePlain : knob_value == 2 ? kStoreStream
+         : knob_value == 3 ? kStoreThrough : default_kind;
 }
 
 // Element traits: how many elements a 16-byte vector holds and how to move between storage and fp32.

@@ -11,7 +11,7 @@
 //   repeat_kv_cache            src/kernels/repeat_kv.cu:10-100
 //
 // Design: one 16-byte vector per lane, a workgroup covers one 4 KiB chunk of the contiguous side,
-// non-temporal stores; k and v go in one launch (the reference issues two).  Rows whose index
+// non-temporal write-through stores; k and v go in one launch (the reference issues two).  Rows whose index
 // would fall outside the destination are skipped instead of written out of bounds.
 #include "isp_common.h"
 
@@ -60,7 +60,7 @@ __global__ __launch_bounds__(kBlock) void transpose_remove_padding_vec(
     unsigned h, c;
     sp.split(vi, h, c);
     const size_t from = ((((size_t)b * head_num + h) * seq_len + s) * seg_vec + c) * 16u;
-    store16_stream(dst + ((size_t)token * row_vec + vi) * 16u, load16_stream(src + from));
+    store16_through(dst + ((size_t)token * row_vec + vi) * 16u, load16_stream(src + from));
 }
 
 __global__ __launch_bounds__(kBlock) void transpose_remove_padding_bytes(
@@ -96,7 +96,7 @@ __global__ __launch_bounds__(kBlock) void concat_kv_vec(
     const int cur = cur_query_length[b];
     const long long row = (long long)history_length[b] + t;
     if ((int)t >= cur || row < 0 || row >= max_seq_len) return;
-    store16_stream(cache + (((size_t)bh * max_seq_len + (size_t)row) * seg_vec + c) * 16u,
+    store16_through(cache + (((size_t)bh * max_seq_len + (size_t)row) * seg_vec + c) * 16u,
                    load16_stream(src + ((size_t)bh * max_q_len * seg_vec + vi) * 16u));
 }
 
@@ -131,7 +131,7 @@ __global__ __launch_bounds__(kBlock) void repeat_kv_vec(
     sp.split(vi, s, c);
     if ((int)s >= context_length[b] || (int)s >= max_seq_len) return;
     const unsigned kvh = h / (unsigned)(head_num / kv_head_num);
-    store16_stream(dst + ((size_t)bh * max_k_len * seg_vec + vi) * 16u,
+    store16_through(dst + ((size_t)bh * max_k_len * seg_vec + vi) * 16u,
                    load16_stream(cache + (((size_t)b * kv_head_num + kvh) * max_seq_len * seg_vec + vi) * 16u));
 }
 

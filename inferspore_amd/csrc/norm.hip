@@ -14,10 +14,10 @@ namespace isp {
 // One row is handled by WPR waves (ROW_THREADS = 64 * WPR lanes); a workgroup has at least 256
 // threads and therefore carries 4 / WPR rows when WPR < 4.  Each lane owns NV 16-byte vectors of
 // the row, strided by ROW_THREADS so that every load instruction of a wave covers 1 KiB of
-// contiguous memory.  NT selects non-temporal stores for the two outputs.
+// contiguous memory.  ST is the store kind of the two outputs (non-temporal by default).
 constexpr int norm_block(int wpr) { return kWave * wpr > kBlock ? kWave * wpr : kBlock; }
 
-template <typename T, int NV, int WPR, bool NT>
+template <typename T, int NV, int WPR, int ST>
 __global__ __launch_bounds__(norm_block(WPR)) void fused_norm_rows(T* __restrict__ residual,
                                                                    T* __restrict__ out,
                                                                    const T* __restrict__ bias,
@@ -67,7 +67,7 @@ __global__ __launch_bounds__(norm_block(WPR)) void fused_norm_rows(T* __restrict
 #pragma unroll
                 for (int e = 0; e < VEC; e++) x[j][e] += r[e];
                 if (flags & ISP_NORM_RESIDUAL_EXCLUDES_BIAS)
-                    store16_sel<NT>(rsd_row + (size_t)vi * VEC, Elem<T>::pack(x[j]));
+                    store16_sel<ST>(rsd_row + (size_t)vi * VEC, Elem<T>::pack(x[j]));
             }
             if (bias) {
                 float b[VEC];
@@ -76,7 +76,7 @@ __global__ __launch_bounds__(norm_block(WPR)) void fused_norm_rows(T* __restrict
                 for (int e = 0; e < VEC; e++) x[j][e] += b[e];
             }
             if (rsd_row && !(flags & ISP_NORM_RESIDUAL_EXCLUDES_BIAS))
-                store16_sel<NT>(rsd_row + (size_t)vi * VEC, Elem<T>::pack(x[j]));
+                store16_sel<ST>(rsd_row + (size_t)vi * VEC, Elem<T>::pack(x[j]));
 #pragma unroll
             for (int e = 0; e < VEC; e++) acc += x[j][e] * x[j][e];
         }
@@ -111,7 +111,7 @@ __global__ __launch_bounds__(norm_block(WPR)) void fused_norm_rows(T* __restrict
             float y[VEC];
 #pragma unroll
             for (int e = 0; e < VEC; e++) y[e] = g[e] * x[j][e] * inv;
-            store16_sel<NT>(out_row + (size_t)vi * VEC, Elem<T>::pack(y));
+            store16_sel<ST>(out_row + (size_t)vi * VEC, Elem<T>::pack(y));
         }
     }
 }
@@ -151,36 +151,36 @@ __global__ __launch_bounds__(kBlock) void fused_norm_generic(T* residual, T* out
     }
 }
 
-template <typename T, int NV, int WPR, bool NT>
+template <typename T, int NV, int WPR, int ST>
 static hipError_t launch_rows(T* residual, T* out, const T* bias, const T* gamma, float eps,
                               int tokens, int hidden, unsigned flags, hipStream_t s) {
     constexpr int BLOCK = norm_block(WPR);
     constexpr int ROWS = BLOCK / (kWave * WPR);
     dim3 grid((unsigned)((tokens + ROWS - 1) / ROWS));
-    hipLaunchKernelGGL((fused_norm_rows<T, NV, WPR, NT>), grid, dim3(BLOCK), 0, s, residual, out,
+    hipLaunchKernelGGL((fused_norm_rows<T, NV, WPR, ST>), grid, dim3(BLOCK), 0, s, residual, out,
                        bias, gamma, eps, tokens, hidden, flags);
     return hipGetLastError();
 }
 
-template <typename T, int WPR, bool NT>
+template <typename T, int WPR, int ST>
 static hipError_t launch_rows_nv(int nv, T* residual, T* out, const T* bias, const T* gamma,
                                  float eps, int tokens, int hidden, unsigned flags, hipStream_t s) {
-    if (nv <= 1) return launch_rows<T, 1, WPR, NT>(residual, out, bias, gamma, eps, tokens, hidden, flags, s);
-    if (nv <= 2) return launch_rows<T, 2, WPR, NT>(residual, out, bias, gamma, eps, tokens, hidden, flags, s);
-    if (nv <= 4) return launch_rows<T, 4, WPR, NT>(residual, out, bias, gamma, eps, tokens, hidden, flags, s);
-    return launch_rows<T, 8, WPR, NT>(residual, out, bias, gamma, eps, tokens, hidden, flags, s);
+    if (nv <= 1) return launch_rows<T, 1, WPR, ST>(residual, out, bias, gamma, eps, tokens, hidden, flags, s);
+    if (nv <= 2) return launch_rows<T, 2, WPR, ST>(residual, out, bias, gamma, eps, tokens, hidden, flags, s);
+    if (nv <= 4) return launch_rows<T, 4, WPR, ST>(residual, out, bias, gamma, eps, tokens, hidden, flags, s);
+    return launch_rows<T, 8, WPR, ST>(residual, out, bias, gamma, eps, tokens, hidden, flags, s);
 }
 
-template <typename T, bool NT>
+template <typename T, int ST>
 static hipError_t launch_rows_wpr(int wpr, int nv, T* residual, T* out, const T* bias,
                                   const T* gamma, float eps, int tokens, int hidden, unsigned flags,
                                   hipStream_t s) {
     switch (wpr) {
-        case 1: return launch_rows_nv<T, 1, NT>(nv, residual, out, bias, gamma, eps, tokens, hidden, flags, s);
-        case 2: return launch_rows_nv<T, 2, NT>(nv, residual, out, bias, gamma, eps, tokens, hidden, flags, s);
-        case 4: return launch_rows_nv<T, 4, NT>(nv, residual, out, bias, gamma, eps, tokens, hidden, flags, s);
-        case 8: return launch_rows_nv<T, 8, NT>(nv, residual, out, bias, gamma, eps, tokens, hidden, flags, s);
-        default: return launch_rows_nv<T, 16, NT>(nv, residual, out, bias, gamma, eps, tokens, hidden, flags, s);
+        case 1: return launch_rows_nv<T, 1, ST>(nv, residual, out, bias, gamma, eps, tokens, hidden, flags, s);
+        case 2: return launch_rows_nv<T, 2, ST>(nv, residual, out, bias, gamma, eps, tokens, hidden, flags, s);
+        case 4: return launch_rows_nv<T, 4, ST>(nv, residual, out, bias, gamma, eps, tokens, hidden, flags, s);
+        case 8: return launch_rows_nv<T, 8, ST>(nv, residual, out, bias, gamma, eps, tokens, hidden, flags, s);
+        default: return launch_rows_nv<T, 16, ST>(nv, residual, out, bias, gamma, eps, tokens, hidden, flags, s);
     }
 }
 
@@ -222,10 +222,14 @@ static int fused_norm(void* residual_, void* out_, const void* bias_, const void
         }
         while (wpr < kMaxWpr && vectors_per_lane(wpr) > kMaxNv) wpr *= 2;
         const int nv = vectors_per_lane(wpr);
-        if (tuning(ISP_TUNE_NORM_STORE) != 1)
-            e = launch_rows_wpr<T, true>(wpr, nv, residual, out, bias, gamma, eps, tokens, hidden, flags, s);
+        // in place on both tensors: plain non-temporal stores measured best (write-through costs 2 %)
+        const int kind = store_kind(tuning(ISP_TUNE_NORM_STORE), kStoreStream);
+        if (kind == kStoreThrough)
+            e = launch_rows_wpr<T, kStoreThrough>(wpr, nv, residual, out, bias, gamma, eps, tokens, hidden, flags, s);
+        else if (kind == kStoreStream)
+            e = launch_rows_wpr<T, kStoreStream>(wpr, nv, residual, out, bias, gamma, eps, tokens, hidden, flags, s);
         else
-            e = launch_rows_wpr<T, false>(wpr, nv, residual, out, bias, gamma, eps, tokens, hidden, flags, s);
+            e = launch_rows_wpr<T, kStorePlain>(wpr, nv, residual, out, bias, gamma, eps, tokens, hidden, flags, s);
     }
     return note_launch(e);
 }

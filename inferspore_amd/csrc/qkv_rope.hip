@@ -54,7 +54,7 @@ __device__ __forceinline__ void rotate_pair(float c, float sn, float x0, float x
 // two stores), evaluates the token's (cos, sin) pairs itself (lane d evaluates pair d) and shares
 // them through a wave-private slice of LDS, so there is no workgroup barrier; waves that only carry
 // v heads skip the evaluation.  grid = (tokens, head groups of 4 waves).
-template <typename T, int HS, bool NT, int WAVES>
+template <typename T, int HS, int ST, int WAVES>
 __global__ __launch_bounds__(kWave * WAVES) void qkv_rope_wave(
     T* __restrict__ q, T* __restrict__ k, T* __restrict__ v, const T* __restrict__ qkv,
     const T* __restrict__ bias, const int32_t* __restrict__ padding_offset,
@@ -154,8 +154,8 @@ __global__ __launch_bounds__(kWave * WAVES) void qkv_rope_wave(
         y0[e] = r ? r0 : x0[e];
         y1[e] = r ? r1 : x1[e];
     }
-    store16_sel<NT>(dst + col, Elem<T>::pack(y0));
-    store16_sel<NT>(dst + HALF + col, Elem<T>::pack(y1));
+    store16_sel<ST>(dst + col, Elem<T>::pack(y0));
+    store16_sel<ST>(dst + HALF + col, Elem<T>::pack(y1));
 }
 
 // Any (even) head size and any alignment: one workgroup per token, one lane per rotation pair.
@@ -352,22 +352,28 @@ static int qkv_rope(void* q_, void* k_, void* v_, const void* qkv_, const void* 
                         (!bias || aligned16(bias));
     dim3 grid((unsigned)token_num), block(kBlock);
     hipError_t e;
-    const bool nt = tuning(ISP_TUNE_QKV_STORE) != 1;
+    const int kind = store_kind(tuning(ISP_TUNE_QKV_STORE), kStoreThrough);
     int waves = tuning(ISP_TUNE_QKV_WAVES);
     if (waves != 1 && waves != 2 && waves != 4) waves = 4;  // 4 measured best (8 and 12 are slower)
-#define ISP_QKV_LAUNCH_1(HS, N, W)                                                                 \
+#define ISP_QKV_LAUNCH_1(HS, K, W)                                                                 \
     do {                                                                                           \
         constexpr int HPB = (kWave / ((HS / 2) / Elem<T>::kVec)) * W;                              \
         dim3 g2((unsigned)token_num, (unsigned)((head_num + 2 * kv_head_num + HPB - 1) / HPB));    \
-        hipLaunchKernelGGL((qkv_rope_wave<T, HS, N, W>), g2, dim3(kWave * W), 0, s, q, k, v, qkv,   \
+        hipLaunchKernelGGL((qkv_rope_wave<T, HS, K, W>), g2, dim3(kWave * W), 0, s, q, k, v, qkv,   \
                            bias, padding_offset, history_length, batch, seq_len, head_num,         \
                            kv_head_num, half_rot, tab);                                            \
     } while (0)
+#define ISP_QKV_LAUNCH_K(HS, W)                                                                    \
+    do {                                                                                           \
+        if (kind == kStoreThrough) ISP_QKV_LAUNCH_1(HS, kStoreThrough, W);                         \
+        else if (kind == kStoreStream) ISP_QKV_LAUNCH_1(HS, kStoreStream, W);                      \
+        else ISP_QKV_LAUNCH_1(HS, kStorePlain, W);                                                 \
+    } while (0)
 #define ISP_QKV_LAUNCH_WAVE(HS)                                                                    \
     do {                                                                                           \
-        if (waves == 1) { if (nt) ISP_QKV_LAUNCH_1(HS, true, 1); else ISP_QKV_LAUNCH_1(HS, false, 1); } \
-        else if (waves == 2) { if (nt) ISP_QKV_LAUNCH_1(HS, true, 2); else ISP_QKV_LAUNCH_1(HS, false, 2); } \
-        else { if (nt) ISP_QKV_LAUNCH_1(HS, true, 4); else ISP_QKV_LAUNCH_1(HS, false, 4); }       \
+        if (waves == 1) ISP_QKV_LAUNCH_K(HS, 1);                                                   \
+        else if (waves == 2) ISP_QKV_LAUNCH_K(HS, 2);                                              \
+        else ISP_QKV_LAUNCH_K(HS, 4);                                                              \
     } while (0)
     const int head_groups_max = 65535 * 4;  // grid.y limit, 4 heads per workgroup at least
     if (vec_ok && head_size == 128 && head_num + 2 * kv_head_num <= head_groups_max) {

@@ -26,7 +26,7 @@ __device__ __forceinline__ float silu_for<float>(float x) { return silu_exact(x)
 template <>
 __device__ __forceinline__ float silu_for<__half>(float x) { return silu_fast(x); }
 
-template <typename T, int UNROLL, bool NT>
+template <typename T, int UNROLL, int ST>
 __global__ __launch_bounds__(kBlock) void swiglu_vec(const T* __restrict__ in, T* __restrict__ out,
                                                      unsigned total_vec, unsigned vec_per_row) {
     constexpr int VEC = Elem<T>::kVec;
@@ -53,7 +53,7 @@ __global__ __launch_bounds__(kBlock) void swiglu_vec(const T* __restrict__ in, T
             Elem<T>::unpack(u[k], b);
 #pragma unroll
             for (int e = 0; e < VEC; e++) y[e] = silu_for<T>(a[e]) * b[e];
-            store16_sel<NT>(out + (size_t)v * VEC, Elem<T>::pack(y));
+            store16_sel<ST>(out + (size_t)v * VEC, Elem<T>::pack(y));
         }
     }
 }
@@ -86,15 +86,22 @@ static int swiglu(const void* in_, void* out_, int tokens, int inter, hipStream_
     if (inter % VEC == 0 && aligned16(in) && aligned16(out) && total_vec < 0xffffffffull) {
         int unroll = tuning(ISP_TUNE_SWIGLU_UNROLL);
         if (unroll != 1 && unroll != 2 && unroll != 4) unroll = 1;
-        const bool nt = tuning(ISP_TUNE_SWIGLU_STORE) != 1;
+        const int kind = store_kind(tuning(ISP_TUNE_SWIGLU_STORE), kStoreStream);
         const size_t per_block = (size_t)kBlock * unroll;
         const dim3 grid((unsigned)((total_vec + per_block - 1) / per_block)), block(kBlock);
         const unsigned nv = (unsigned)total_vec, vpr = (unsigned)(inter / VEC);
-#define ISP_SWIGLU_LAUNCH(U, N) \
-    hipLaunchKernelGGL((swiglu_vec<T, U, N>), grid, block, 0, s, in, out, nv, vpr)
-        if (unroll == 1) { if (nt) ISP_SWIGLU_LAUNCH(1, true); else ISP_SWIGLU_LAUNCH(1, false); }
-        else if (unroll == 2) { if (nt) ISP_SWIGLU_LAUNCH(2, true); else ISP_SWIGLU_LAUNCH(2, false); }
-        else { if (nt) ISP_SWIGLU_LAUNCH(4, true); else ISP_SWIGLU_LAUNCH(4, false); }
+#define ISP_SWIGLU_LAUNCH(U, K) \
+    hipLaunchKernelGGL((swiglu_vec<T, U, K>), grid, block, 0, s, in, out, nv, vpr)
+#define ISP_SWIGLU_KIND(U)                                               \
+    do {                                                                 \
+        if (kind == kStoreThrough) ISP_SWIGLU_LAUNCH(U, kStoreThrough);  \
+        else if (kind == kStoreStream) ISP_SWIGLU_LAUNCH(U, kStoreStream); \
+        else ISP_SWIGLU_LAUNCH(U, kStorePlain);                          \
+    } while (0)
+        if (unroll == 1) ISP_SWIGLU_KIND(1);
+        else if (unroll == 2) ISP_SWIGLU_KIND(2);
+        else ISP_SWIGLU_KIND(4);
+#undef ISP_SWIGLU_KIND
 #undef ISP_SWIGLU_LAUNCH
         e = hipGetLastError();
     } else {
