@@ -29,22 +29,22 @@ import time
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published peak
 
 # HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE and WRITE_SIZE in separate runs, each
-# scaled by what the same counter reads for isp_calibration_copy of known size: x1.9987 and x0.9986).
+# scaled by what the same counter reads for isp_calibration_copy of known size: x1.9986 and x1.0000).
 # The summary of those runs is profiles/all_kernels_benchmark_shapes.hbm_traffic_pmc.txt.
 MEASURED_TRAFFIC_BYTES = {
-    "fused_add_bias_residual_rmsnorm_f16_2048x4096": 67220187,
-    "rmsnorm_f32_64x4096": 2256656,
-    "rmsnorm_f32_16384x4096": 536490518,
-    "embedding_f16_8192x4096_v32000": 133616596,
-    "qkv_bias_rope_transpose_f16_b8_s512": 146643388,
-    "swiglu_f16_prefill_8192x11008": 540601380,
-    "swiglu_f16_decode_256x11008": 16921499,
-    "transpose_remove_padding_f16_b8_s512": 48954297,
-    "concat_kv_cache_f16_b8_q512_S1024": 97464471,
-    "repeat_kv_cache_f16_b8_k512_S1024": 97478542,
-    "rope_decode_f16_1x96x128": 49363,
+    "fused_add_bias_residual_rmsnorm_f16_2048x4096": 67266959,
+    "rmsnorm_f32_64x4096": 2252960,
+    "rmsnorm_f32_16384x4096": 536949649,
+    "embedding_f16_8192x4096_v32000": 133248695,
+    "qkv_bias_rope_transpose_f16_b8_s512": 146749274,
+    "swiglu_f16_prefill_8192x11008": 540835621,
+    "swiglu_f16_decode_256x11008": 16928861,
+    "transpose_remove_padding_f16_b8_s512": 48988181,
+    "concat_kv_cache_f16_b8_q512_S1024": 97531754,
+    "repeat_kv_cache_f16_b8_k512_S1024": 97546079,
+    "rope_decode_f16_1x96x128": 49384,
     "calibration_copy_64MiB_traffic": 67108864,
-    "calibration_copy_512MiB_traffic": 536471488,
+    "calibration_copy_512MiB_traffic": 536697980,
 }
 
 
@@ -123,7 +123,7 @@ def make_workloads(torch, lib, stream_handle, rotate):
             wpr *= 2
         nv = -(-nvec // (64 * wpr))
         nv = 1 if nv <= 1 else 2 if nv <= 2 else 4 if nv <= 4 else 8
-        w.kernel = "isp::fused_norm_rows<%s, %d, %d, true>" % ("__half" if es == 2 else "float", nv, wpr)
+        w.kernel = "isp::fused_norm_rows<%s, %d, %d, 1>" % ("__half" if es == 2 else "float", nv, wpr)
         if fused:
             fn = getattr(lib, "isp_fused_add_bias_residual_rmsnorm_" + sfx)
             w.bind(fn, [(ress[j].data_ptr(), outs[j].data_ptr(), bias.data_ptr(), gamma.data_ptr(), 1e-5, tokens,
@@ -148,7 +148,7 @@ def make_workloads(torch, lib, stream_handle, rotate):
         w = Workload()
         tokens, hidden, vocab = 8192, 4096, 32000
         w.name, w.dtype, w.tokens = "embedding_f16_8192x4096_v32000", "f16", tokens
-        w.kernel = "isp::gather_chunks_vec<true>"
+        w.kernel = "isp::gather_chunks_vec<2>"
         w.bytes_per_launch = 2 * tokens * hidden * 2 + tokens * 4
         table = (0.02 * torch.randn((vocab, hidden), device=dev)).to(torch.float16)
         R = w.sets_for(tokens * hidden * 2, rotate)
@@ -168,7 +168,7 @@ def make_workloads(torch, lib, stream_handle, rotate):
         lens = torch.randint(256, 513, (batch,), generator=g, dtype=torch.int32)
         tokens = int(lens.sum())
         w.name, w.dtype, w.tokens = "qkv_bias_rope_transpose_f16_b8_s512", "f16", tokens
-        w.kernel = "isp::qkv_rope_wave<__half, 128, true>"
+        w.kernel = "isp::qkv_rope_wave<__half, 128, 2, 4>"
         w.bytes_per_launch = tokens * (2 * (hn + 2 * kvn) * hs * 2 + 4) + (hn + 2 * kvn) * hs * 2 + 2 * batch * 4
         lens_d = lens.to(dev)
         po = torch.zeros((batch, seq), device=dev, dtype=torch.int32)
@@ -195,7 +195,7 @@ def make_workloads(torch, lib, stream_handle, rotate):
         w = Workload()
         inter = 11008
         w.name, w.dtype, w.tokens = "swiglu_f16_%s_%dx%d" % (tag, tokens, inter), "f16", tokens
-        w.kernel = "isp::swiglu_vec<__half, 1, true>"
+        w.kernel = "isp::swiglu_vec<__half, 1, 1>"
         w.bytes_per_launch = tokens * 3 * inter * 2
         R = w.sets_for(w.bytes_per_launch, rotate)
         ins = [torch.randn((tokens, 2, inter), device=dev).to(torch.float16) for _ in range(R)]
