@@ -73,11 +73,6 @@ __global__ __launch_bounds__(kWave * WAVES) void qkv_rope_wave(
     const int lane = threadIdx.x % kWave;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     const int token = (int)blockIdx.x;
-    const long long p = (long long)token + (long long)padding_offset[token];
-    if (p < 0 || p >= (long long)batch * (long long)seq_len) return;  // wave-uniform
-    const int b = (int)(p / seq_len);
-    const int s = (int)(p % seq_len);
-
     const int g = lane % G;
     const int slot = lane / G;
     const int qkv_heads = head_num + 2 * kv_head_num;
@@ -88,6 +83,9 @@ __global__ __launch_bounds__(kWave * WAVES) void qkv_rope_wave(
     const int col = g * VEC;
     const T* src = qkv + ((size_t)token * (size_t)qkv_heads + (live ? h : 0)) * HS;
 
+    // The source address depends on the token index only, so the streamed loads are issued before
+    // the destination (padding_offset -> batch row -> history) is known: the dependent scalar
+    // loads then overlap the HBM latency instead of preceding it.
     vec16 lo, hi, blo, bhi;
     if (live) {
         lo = load16_stream(src + col);
@@ -97,6 +95,10 @@ __global__ __launch_bounds__(kWave * WAVES) void qkv_rope_wave(
             bhi = load16(bias + (size_t)h * HS + HALF + col);
         }
     }
+    const long long p = (long long)token + (long long)padding_offset[token];
+    if (p < 0 || p >= (long long)batch * (long long)seq_len) return;  // wave-uniform
+    const int b = (int)(p / seq_len);
+    const int s = (int)(p % seq_len);
 
     float c[VEC], sn[VEC];
 #pragma unroll
