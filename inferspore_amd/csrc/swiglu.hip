@@ -83,7 +83,8 @@ static int swiglu(const void* in_, void* out_, int tokens, int inter, hipStream_
     const size_t total = (size_t)tokens * (size_t)inter;
     const size_t total_vec = total / VEC;
     hipError_t e;
-    if (inter % VEC == 0 && aligned16(in) && aligned16(out) && total_vec < 0xffffffffull) {
+    // 32-bit vector indices in the kernel: leave room for the last workgroup's overshoot
+    if (inter % VEC == 0 && aligned16(in) && aligned16(out) && total_vec < 0xffff0000ull) {
         int unroll = tuning(ISP_TUNE_SWIGLU_UNROLL);
         if (unroll != 1 && unroll != 2 && unroll != 4) unroll = 1;
         const int kind = store_kind(tuning(ISP_TUNE_SWIGLU_STORE), kStoreStream);
