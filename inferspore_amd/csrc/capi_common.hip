@@ -15,6 +15,20 @@ int note_launch(hipError_t e) {
 
 static int g_tuning[ISP_TUNE_COUNT] = {0};
 
+int resident_waves() {
+    constexpr int kMaxDevices = 64;
+    static int cached[kMaxDevices] = {0};  // written with the same value by every thread
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 256 * 32;
+    if (cached[dev] == 0) {
+        int cus = 0;
+        if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+            cus = 256;
+        cached[dev] = cus * 32;  // 4 SIMDs x 8 wavefronts per compute unit
+    }
+    return cached[dev];
+}
+
 int tuning(int knob) { return (knob >= 0 && knob < ISP_TUNE_COUNT) ? g_tuning[knob] : 0; }
 
 }  // namespace isp

@@ -20,6 +20,9 @@ int note_launch(hipError_t e);
 // Current value of a tuning knob (isp_tuning_set); 0 means "automatic" for every knob.
 int tuning(int knob);
 
+// Wavefronts the current device holds at once (compute units x 32), cached per device.
+int resident_waves();
+
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 #define ISP_REQUIRE_PTR(p)                   \

@@ -213,12 +213,30 @@ static int fused_norm(void* residual_, void* out_, const void* bias_, const void
         auto vectors_per_lane = [nvec](int w) { return (nvec + kWave * w - 1) / (kWave * w); };
         int wpr = tuning(ISP_TUNE_NORM_WAVES_PER_ROW);
         if (wpr != 1 && wpr != 2 && wpr != 4 && wpr != 8 && wpr != 16) {
-            // automatic: the fewest waves per row that leave at most 2 vectors per lane; when there
-            // are too few rows to occupy the machine (4 waves on each of 1024 SIMDs), split rows
-            // further, down to one vector per lane
+            // Automatic, from sweeps over 512..16384 rows of 2048..8192 elements, both types:
+            //  * streaming regime (several rounds of waves): about two 16-byte loads in flight
+            //    per lane, i.e. waves per row = vectors x operand streams / 128, rounded to the
+            //    nearest power of two;
+            //  * if that needs more waves than the device holds at once, but fewer waves per row
+            //    (at most 4 vectors per lane) fit the whole launch into a single round, take the
+            //    single round: every load is then issued at kernel start (5-10 % faster);
+            //  * few rows: split rows further, down to one vector per lane, to occupy the machine.
+            const int streams = residual ? 2 : 1;
+            const int want = nvec * streams;  // 16-byte loads per row
             wpr = 1;
-            while (wpr < kMaxWpr && vectors_per_lane(wpr) > 2) wpr *= 2;
-            while (wpr < kMaxWpr && vectors_per_lane(wpr) > 1 && (long long)tokens * wpr < 4096) wpr *= 2;
+            while (wpr < kMaxWpr && 3 * kWave * wpr < want) wpr *= 2;  // 2^round(log2(want / 128))
+            const long long capacity = resident_waves();
+            if ((long long)tokens * wpr > capacity) {
+                for (int w = wpr / 2; w >= 1; w /= 2) {
+                    if ((long long)tokens * w <= capacity) {
+                        if (vectors_per_lane(w) <= 4) wpr = w;
+                        break;
+                    }
+                }
+            } else {
+                while (wpr < kMaxWpr && vectors_per_lane(wpr) > 1 && (long long)tokens * wpr < capacity / 2)
+                    wpr *= 2;
+            }
         }
         while (wpr < kMaxWpr && vectors_per_lane(wpr) > kMaxNv) wpr *= 2;
         const int nv = vectors_per_lane(wpr);
