@@ -279,10 +279,21 @@ __global__ __launch_bounds__(kBlock) void rope_decode_generic(T* qkv, int head_n
     }
 }
 
+// base^(2d/rot) with the C library's powf.  A model calls with one (rot, base) over and over, and
+// 128 powf cost about as much host time as the whole launch of a decode step, so each host thread
+// keeps the table of its last call.
 static void fill_divisors(RopeDivisors& tab, int rot, float base) {
-    const int half_rot = rot / 2;
-    for (int d = 0; d < kMaxHalfRot; d++)
-        tab.div[d] = d < half_rot ? powf(base, (float)(2 * d) / (float)rot) : 1.0f;
+    static thread_local RopeDivisors cached;
+    static thread_local int cached_rot = -1;
+    static thread_local float cached_base = 0.0f;
+    if (cached_rot != rot || cached_base != base) {
+        const int half_rot = rot / 2;
+        for (int d = 0; d < kMaxHalfRot; d++)
+            cached.div[d] = d < half_rot ? powf(base, (float)(2 * d) / (float)rot) : 1.0f;
+        cached_rot = rot;
+        cached_base = base;
+    }
+    tab = cached;
 }
 
 template <typename T>
