@@ -67,16 +67,17 @@ __global__ __launch_bounds__(kBlock) void gather_chunks_vec(const int32_t* __res
     store16_sel<ST>(out + (size_t)row * row_bytes + (size_t)v * 16u, buf);
 }
 
-// Rows that are not a whole number of aligned 16-byte vectors: one workgroup per row, byte copies.
-__global__ __launch_bounds__(kBlock) void gather_rows_bytes(const int32_t* ids, char* out,
-                                                            const char* table, int tokens,
-                                                            size_t row_bytes, int vocab) {
+// Rows that are not a whole number of aligned 16-byte vectors: one workgroup per row, copied in units
+// of U (the element size when the pointers allow it, bytes otherwise).
+template <typename U>
+__global__ __launch_bounds__(kBlock) void gather_rows_units(const int32_t* ids, U* out, const U* table,
+                                                            int tokens, size_t row_units, int vocab) {
     const int row = blockIdx.x;
     const int id = ids[row];
     const bool in_range = vocab <= 0 || (id >= 0 && id < vocab);
-    const char* src = table + (size_t)(in_range ? id : 0) * row_bytes;
-    char* dst = out + (size_t)row * row_bytes;
-    for (size_t i = threadIdx.x; i < row_bytes; i += kBlock) dst[i] = in_range ? src[i] : (char)0;
+    const U* src = table + (size_t)(in_range ? id : 0) * row_units;
+    U* dst = out + (size_t)row * row_units;
+    for (size_t i = threadIdx.x; i < row_units; i += kBlock) dst[i] = in_range ? src[i] : (U)0;
 }
 
 template <int ST>
@@ -116,9 +117,17 @@ static int embedding(const int32_t* ids, void* out, const void* table, int token
         else launch_gather<kStorePlain>(variant, ids, o, t, tokens, row_vec, vocab, s);
         e = hipGetLastError();
     } else {
-        hipLaunchKernelGGL(gather_rows_bytes, dim3((unsigned)tokens), dim3(kBlock), 0, s, ids,
-                           static_cast<char*>(out), static_cast<const char*>(table), tokens,
-                           row_bytes, vocab);
+        const dim3 grid((unsigned)tokens), block(kBlock);
+        const int unit = copy_unit(row_bytes, out, table);
+        if (unit == 4)
+            hipLaunchKernelGGL(gather_rows_units<uint32_t>, grid, block, 0, s, ids, static_cast<uint32_t*>(out),
+                               static_cast<const uint32_t*>(table), tokens, row_bytes / 4, vocab);
+        else if (unit == 2)
+            hipLaunchKernelGGL(gather_rows_units<uint16_t>, grid, block, 0, s, ids, static_cast<uint16_t*>(out),
+                               static_cast<const uint16_t*>(table), tokens, row_bytes / 2, vocab);
+        else
+            hipLaunchKernelGGL(gather_rows_units<uint8_t>, grid, block, 0, s, ids, static_cast<uint8_t*>(out),
+                               static_cast<const uint8_t*>(table), tokens, row_bytes, vocab);
         e = hipGetLastError();
     }
     return note_launch(e);

@@ -25,6 +25,15 @@ int resident_waves();
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
+// Widest unit (4, 2 or 1 bytes) that divides `bytes` and the addresses of all the given pointers:
+// the copy width of the fallback kernels for rows that are not whole aligned 16-byte vectors.
+template <typename... P>
+inline int copy_unit(size_t bytes, const P*... ptrs) {
+    uintptr_t bits = (uintptr_t)bytes;
+    ((bits |= reinterpret_cast<uintptr_t>(ptrs)), ...);
+    return (bits & 3u) == 0 ? 4 : (bits & 1u) == 0 ? 2 : 1;
+}
+
 #define ISP_REQUIRE_PTR(p)                   \
     do {                                     \
         if ((p) == nullptr) return ISP_ERR_NULL_POINTER; \

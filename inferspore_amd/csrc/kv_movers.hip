@@ -63,17 +63,20 @@ __global__ __launch_bounds__(kBlock) void transpose_remove_padding_vec(
     store16_through(dst + ((size_t)token * row_vec + vi) * 16u, load16_stream(src + from));
 }
 
-__global__ __launch_bounds__(kBlock) void transpose_remove_padding_bytes(
-    const char* src, const int32_t* padding_offset, char* dst, int batch, int head_num, int seq_len,
-    size_t seg_bytes) {
+// Fallbacks for head rows that are not whole aligned 16-byte vectors: copies in units of U (4, 2 or 1
+// bytes, the widest the sizes and addresses allow); `seg` counts units per head row.
+template <typename U>
+__global__ __launch_bounds__(kBlock) void transpose_remove_padding_units(
+    const U* src, const int32_t* padding_offset, U* dst, int batch, int head_num, int seq_len,
+    size_t seg) {
     const unsigned token = blockIdx.x;
     const long long p = (long long)token + (long long)padding_offset[token];
     if (p < 0 || p >= (long long)batch * seq_len) return;
     const size_t b = (size_t)(p / seq_len), s = (size_t)(p % seq_len);
-    const size_t row = (size_t)head_num * seg_bytes;
+    const size_t row = (size_t)head_num * seg;
     for (size_t i = threadIdx.x; i < row; i += kBlock) {
-        const size_t h = i / seg_bytes, c = i % seg_bytes;
-        dst[(size_t)token * row + i] = src[((b * head_num + h) * seq_len + s) * seg_bytes + c];
+        const size_t h = i / seg, c = i % seg;
+        dst[(size_t)token * row + i] = src[((b * head_num + h) * seq_len + s) * seg + c];
     }
 }
 
@@ -100,18 +103,19 @@ __global__ __launch_bounds__(kBlock) void concat_kv_vec(
                    load16_stream(src + ((size_t)bh * max_q_len * seg_vec + vi) * 16u));
 }
 
-__global__ __launch_bounds__(kBlock) void concat_kv_bytes(
-    const char* k_src, const char* v_src, char* k_cache, char* v_cache,
+template <typename U>
+__global__ __launch_bounds__(kBlock) void concat_kv_units(
+    const U* k_src, const U* v_src, U* k_cache, U* v_cache,
     const int32_t* cur_query_length, const int32_t* history_length, int kv_head_num, int max_q_len,
-    int max_seq_len, size_t seg_bytes) {
-    const char* src = blockIdx.z == 0 ? k_src : v_src;
-    char* cache = blockIdx.z == 0 ? k_cache : v_cache;
+    int max_seq_len, size_t seg) {
+    const U* src = blockIdx.z == 0 ? k_src : v_src;
+    U* cache = blockIdx.z == 0 ? k_cache : v_cache;
     const unsigned bh = blockIdx.y, b = bh / kv_head_num, t = blockIdx.x;
     const long long row = (long long)history_length[b] + t;
     if ((int)t >= cur_query_length[b] || row < 0 || row >= max_seq_len) return;
-    for (size_t i = threadIdx.x; i < seg_bytes; i += kBlock)
-        cache[((size_t)bh * max_seq_len + (size_t)row) * seg_bytes + i] =
-            src[((size_t)bh * max_q_len + t) * seg_bytes + i];
+    for (size_t i = threadIdx.x; i < seg; i += kBlock)
+        cache[((size_t)bh * max_seq_len + (size_t)row) * seg + i] =
+            src[((size_t)bh * max_q_len + t) * seg + i];
 }
 
 // dst[b, h, s, :] = cache[b, h / rep, s, :] for s < context_length[b]; blockIdx.z selects k / v.
@@ -135,18 +139,19 @@ __global__ __launch_bounds__(kBlock) void repeat_kv_vec(
                    load16_stream(cache + (((size_t)b * kv_head_num + kvh) * max_seq_len * seg_vec + vi) * 16u));
 }
 
-__global__ __launch_bounds__(kBlock) void repeat_kv_bytes(
-    const char* k_cache, const char* v_cache, char* k_dst, char* v_dst,
+template <typename U>
+__global__ __launch_bounds__(kBlock) void repeat_kv_units(
+    const U* k_cache, const U* v_cache, U* k_dst, U* v_dst,
     const int32_t* context_length, int head_num, int kv_head_num, int max_seq_len, int max_k_len,
-    size_t seg_bytes) {
-    const char* cache = blockIdx.z == 0 ? k_cache : v_cache;
-    char* dst = blockIdx.z == 0 ? k_dst : v_dst;
+    size_t seg) {
+    const U* cache = blockIdx.z == 0 ? k_cache : v_cache;
+    U* dst = blockIdx.z == 0 ? k_dst : v_dst;
     const unsigned bh = blockIdx.y, b = bh / head_num, h = bh % head_num, s = blockIdx.x;
     if ((int)s >= context_length[b] || (int)s >= max_seq_len) return;
     const unsigned kvh = h / (unsigned)(head_num / kv_head_num);
-    for (size_t i = threadIdx.x; i < seg_bytes; i += kBlock)
-        dst[((size_t)bh * max_k_len + s) * seg_bytes + i] =
-            cache[(((size_t)b * kv_head_num + kvh) * max_seq_len + s) * seg_bytes + i];
+    for (size_t i = threadIdx.x; i < seg; i += kBlock)
+        dst[((size_t)bh * max_k_len + s) * seg + i] =
+            cache[(((size_t)b * kv_head_num + kvh) * max_seq_len + s) * seg + i];
 }
 
 constexpr long long kMaxGridYZ = 65535;
@@ -169,9 +174,16 @@ static int transpose_remove_padding(const void* src, const int32_t* padding_offs
                            static_cast<const char*>(src), padding_offset, static_cast<char*>(dst),
                            batch, head_num, seq_len, make_split(seg_vec), (unsigned)chunks);
     } else {
-        hipLaunchKernelGGL(transpose_remove_padding_bytes, dim3((unsigned)token_num), dim3(kBlock), 0,
-                           s, static_cast<const char*>(src), padding_offset, static_cast<char*>(dst),
-                           batch, head_num, seq_len, seg);
+        const dim3 grid((unsigned)token_num), block(kBlock);
+#define ISP_LAUNCH_UNITS(U)                                                                        \
+    hipLaunchKernelGGL(transpose_remove_padding_units<U>, grid, block, 0, s,                        \
+                       static_cast<const U*>(src), padding_offset, static_cast<U*>(dst), batch,     \
+                       head_num, seq_len, seg / sizeof(U))
+        const int unit = copy_unit(seg, src, dst);
+        if (unit == 4) ISP_LAUNCH_UNITS(uint32_t);
+        else if (unit == 2) ISP_LAUNCH_UNITS(uint16_t);
+        else ISP_LAUNCH_UNITS(uint8_t);
+#undef ISP_LAUNCH_UNITS
     }
     return note_launch(hipGetLastError());
 }
@@ -205,9 +217,17 @@ static int concat_kv(const void* k_src, const void* v_src, void* k_cache, void* 
         hipLaunchKernelGGL(concat_kv_vec, grid, dim3(kBlock), 0, s, ks, vs, kc, vc, cur_query_length,
                            history_length, kv_head_num, max_q_len, max_seq_len, make_split(seg_vec));
     } else {
-        dim3 grid((unsigned)max_q_len, (unsigned)(batch * kv_head_num), 2);
-        hipLaunchKernelGGL(concat_kv_bytes, grid, dim3(kBlock), 0, s, ks, vs, kc, vc, cur_query_length,
-                           history_length, kv_head_num, max_q_len, max_seq_len, seg);
+        const dim3 grid((unsigned)max_q_len, (unsigned)(batch * kv_head_num), 2), block(kBlock);
+#define ISP_LAUNCH_UNITS(U)                                                                        \
+    hipLaunchKernelGGL(concat_kv_units<U>, grid, block, 0, s, reinterpret_cast<const U*>(ks),       \
+                       reinterpret_cast<const U*>(vs), reinterpret_cast<U*>(kc),                    \
+                       reinterpret_cast<U*>(vc), cur_query_length, history_length, kv_head_num,     \
+                       max_q_len, max_seq_len, seg / sizeof(U))
+        const int unit = copy_unit(seg, ks, vs, kc, vc);
+        if (unit == 4) ISP_LAUNCH_UNITS(uint32_t);
+        else if (unit == 2) ISP_LAUNCH_UNITS(uint16_t);
+        else ISP_LAUNCH_UNITS(uint8_t);
+#undef ISP_LAUNCH_UNITS
     }
     return note_launch(hipGetLastError());
 }
@@ -240,9 +260,17 @@ static int repeat_kv(const void* k_cache, const void* v_cache, void* k_dst, void
         hipLaunchKernelGGL(repeat_kv_vec, grid, dim3(kBlock), 0, s, kc, vc, kd, vd, context_length,
                            head_num, kv_head_num, max_seq_len, max_k_len, make_split(seg_vec));
     } else {
-        dim3 grid((unsigned)max_k_len, (unsigned)(batch * head_num), 2);
-        hipLaunchKernelGGL(repeat_kv_bytes, grid, dim3(kBlock), 0, s, kc, vc, kd, vd, context_length,
-                           head_num, kv_head_num, max_seq_len, max_k_len, seg);
+        const dim3 grid((unsigned)max_k_len, (unsigned)(batch * head_num), 2), block(kBlock);
+#define ISP_LAUNCH_UNITS(U)                                                                        \
+    hipLaunchKernelGGL(repeat_kv_units<U>, grid, block, 0, s, reinterpret_cast<const U*>(kc),       \
+                       reinterpret_cast<const U*>(vc), reinterpret_cast<U*>(kd),                    \
+                       reinterpret_cast<U*>(vd), context_length, head_num, kv_head_num,             \
+                       max_seq_len, max_k_len, seg / sizeof(U))
+        const int unit = copy_unit(seg, kc, vc, kd, vd);
+        if (unit == 4) ISP_LAUNCH_UNITS(uint32_t);
+        else if (unit == 2) ISP_LAUNCH_UNITS(uint16_t);
+        else ISP_LAUNCH_UNITS(uint8_t);
+#undef ISP_LAUNCH_UNITS
     }
     return note_launch(hipGetLastError());
 }

@@ -121,3 +121,88 @@ def test_kv_cache_append_skips_rows_past_the_cache_end(isp):
     isp.concat_kv_cache(k_src, k_src, 0, cur, hist, cache_k, cache_v)
     torch.cuda.synchronize()
     assert torch.all(cache_k[0, 0, :, 4:6] == 1) and torch.all(cache_k[0, 0, :, :4] == 0)
+
+
+# ------------------------------------------------------------------ fallback copy widths (4, 2, 1 bytes)
+@pytest.mark.parametrize("shift", [0, 4, 2, 1])
+def test_fallback_copy_units_through_raw_pointers(isp, shift):
+    """Rows that are not whole aligned 16-byte vectors are copied in the widest unit the addresses allow.
+    `shift` moves every buffer off its 16-byte alignment by that many bytes (0: only the row size is odd),
+    so the 4-, 2- and 1-byte kernels all run; the data are bytes, checked against numpy indexing."""
+    from inferspore_amd import capi
+    lib = capi.lib()
+    st = torch.cuda.current_stream().cuda_stream
+    rng = np.random.default_rng(90 + shift)
+
+    def on_device(a):
+        """Copies a byte array to the device at `shift` bytes past an aligned address."""
+        buf = torch.zeros(a.size + 64, dtype=torch.uint8, device="cuda")
+        view = buf[shift:shift + a.size]
+        view.copy_(torch.from_numpy(a.reshape(-1)))
+        assert view.data_ptr() % 16 == shift % 16
+        return buf, view
+
+    # gather: rows of 10 fp16 elements = 20 bytes (4-byte units at shift 0 and 4, 2 at 2, 1 at 1)
+    tokens, vocab, hidden = 29, 17, 10
+    table = rng.integers(0, 256, (vocab, hidden * 2), dtype=np.uint8)
+    ids = rng.integers(0, vocab, tokens).astype(np.int32)
+    _, d_table = on_device(table)
+    _, d_out = on_device(np.zeros((tokens, hidden * 2), np.uint8))
+    d_ids = torch.from_numpy(ids).cuda()
+    say("gather through raw pointers, shift %d" % shift)
+    capi.check(lib.isp_embedding_f16(d_ids.data_ptr(), d_out.data_ptr(), d_table.data_ptr(), tokens, hidden, vocab, st),
+               "isp_embedding_f16")
+    assert np.array_equal(d_out.cpu().numpy().reshape(tokens, hidden * 2), table[ids])
+
+    # movers: head rows of 6 fp16 elements = 12 bytes
+    batch, heads, seq, hs = 3, 2, 6, 6
+    seg = hs * 2
+    lens = np.array([6, 2, 4], np.int32)
+    src = rng.integers(0, 256, (batch, heads, seq, seg), dtype=np.uint8)
+    tokens = int(lens.sum())
+    po = np.concatenate([np.full(n, b * seq - lens[:b].sum(), np.int32) for b, n in enumerate(lens)])
+    _, d_src = on_device(src)
+    _, d_dst = on_device(np.zeros((tokens, heads, seg), np.uint8))
+    d_po = torch.from_numpy(po).cuda()
+    say("transpose-out through raw pointers, shift %d" % shift)
+    capi.check(lib.isp_transpose_remove_padding_f16(d_src.data_ptr(), d_po.data_ptr(), d_dst.data_ptr(), batch, heads,
+                                                    seq, hs, tokens, st), "isp_transpose_remove_padding_f16")
+    p = np.arange(tokens) + po
+    exp = src[p // seq, :, p % seq, :]
+    assert np.array_equal(d_dst.cpu().numpy().reshape(tokens, heads, seg), exp)
+
+    max_seq = 9
+    hist = np.array([1, 7, 0], np.int32)
+    ksrc, vsrc = src, src[::-1].copy()
+    kc0 = rng.integers(0, 256, (batch, heads, max_seq, seg), dtype=np.uint8)
+    vc0 = rng.integers(0, 256, (batch, heads, max_seq, seg), dtype=np.uint8)
+    _, d_ks = on_device(ksrc)
+    _, d_vs = on_device(vsrc)
+    _, d_kc = on_device(kc0)
+    _, d_vc = on_device(vc0)
+    d_lens, d_hist = torch.from_numpy(lens).cuda(), torch.from_numpy(hist).cuda()
+    say("KV append through raw pointers, shift %d" % shift)
+    capi.check(lib.isp_concat_kv_cache_f16(d_ks.data_ptr(), d_vs.data_ptr(), d_kc.data_ptr(), d_vc.data_ptr(), 0,
+                                           d_lens.data_ptr(), d_hist.data_ptr(), batch, heads, seq, max_seq, hs, st),
+               "isp_concat_kv_cache_f16")
+    for got, s_, c0 in ((d_kc, ksrc, kc0), (d_vc, vsrc, vc0)):
+        exp = c0.copy()
+        for b in range(batch):
+            n = min(int(lens[b]), max_seq - int(hist[b]))
+            exp[b, :, hist[b]:hist[b] + n] = s_[b, :, :n]
+        assert np.array_equal(got.cpu().numpy().reshape(exp.shape), exp)
+
+    ctx = np.array([9, 3, 5], np.int32)
+    max_k = 9
+    _, d_kd = on_device(np.full((batch, heads, max_k, seg), 7, np.uint8))
+    _, d_vd = on_device(np.full((batch, heads, max_k, seg), 7, np.uint8))
+    d_ctx = torch.from_numpy(ctx).cuda()
+    say("KV broadcast through raw pointers, shift %d" % shift)
+    capi.check(lib.isp_repeat_kv_cache_f16(d_kc.data_ptr(), d_vc.data_ptr(), d_kd.data_ptr(), d_vd.data_ptr(), 0,
+                                           d_ctx.data_ptr(), batch, heads, heads, max_seq, max_k, hs, st),
+               "isp_repeat_kv_cache_f16")
+    kc_now = d_kc.cpu().numpy().reshape(batch, heads, max_seq, seg)
+    got = d_kd.cpu().numpy().reshape(batch, heads, max_k, seg)
+    for b in range(batch):
+        assert np.array_equal(got[b, :, :ctx[b]], kc_now[b, :, :ctx[b]])
+        assert (got[b, :, ctx[b]:] == 7).all()
