@@ -19,7 +19,9 @@
  *   - pointers documented "may be NULL" are optional operands; any other NULL pointer gives
  *     ISP_ERR_NULL_POINTER (unless the call has no work to do: zero tokens returns ISP_OK first);
  *   - 16-byte aligned pointers and vector-friendly extents take the fast 128-bit path; anything
- *     else is routed to a slower scalar kernel with identical results.
+ *     else is routed to a slower scalar kernel with identical results.  Tensor pointers must be
+ *     aligned to their element (2 bytes for `_f16`, 4 for `_f32`, 4 for the int32 arrays); the
+ *     pure movers (gather, transpose-out, KV append / broadcast) accept any byte address;
  */
 #ifndef INFERSPORE_AMD_H
 #define INFERSPORE_AMD_H
