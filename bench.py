@@ -607,6 +607,22 @@ def main():
 
     results = run_all(True)
     head = results[0]
+    # The practical ceiling of this device for a read+write stream, from the two plain copies of
+    # this very run: time = fixed + bytes / rate.  Each kernel is also priced against the copy of
+    # equal algorithmic bytes ("vs_copy" = copy-model time / kernel time; 1.0 = at the ceiling).
+    by_name = {r["workload"]: r for r in results}
+    c_small, c_big = by_name.get("calibration_copy_64MiB_traffic"), by_name.get("calibration_copy_512MiB_traffic")
+    copy_model = None
+    if c_small and c_big:
+        rate = (c_big["algorithmic_bytes"] - c_small["algorithmic_bytes"]) / (
+            c_big["ms_per_launch_events"] - c_small["ms_per_launch_events"])          # bytes per ms
+        fixed = c_small["ms_per_launch_events"] - c_small["algorithmic_bytes"] / rate  # ms
+        copy_model = {"fixed_us": fixed * 1e3, "asymptotic_GBps": rate / 1e6,
+                      "form": "copy_time = fixed_us + bytes / asymptotic rate"}
+        for r in results:
+            t = fixed + r["algorithmic_bytes"] / rate
+            r["copy_model_ms"] = t
+            r["vs_copy"] = t / r["ms_per_launch_events"]
     line = {
         "metric": "HBM GB/s & % of peak per fused kernel at LLaMA-2-7B shapes; tokens/sec",
         "value": head["GBps"], "unit": "GB/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
@@ -619,11 +635,12 @@ def main():
                          avg_launch_ms=head["ms_per_launch_events"]),
         "kernels": results,
     }
+    if copy_model:
+        line["copy_ceiling"] = copy_model
     if not a.only:
         layer = context_layer_record(torch, a.steps, a.warmup, stream)
         own = {"qkv_bias_rope_transpose_f16_b8_s512": 1, "concat_kv_cache_f16_b8_q512_S1024": 1,
                "repeat_kv_cache_f16_b8_k512_S1024": 1, "transpose_remove_padding_f16_b8_s512": 1}
-        by_name = {r["workload"]: r for r in results}
         tokens = layer["valid_tokens"]
         # fused norm (x2) and SwiGLU run on `tokens` rows here; scale their measured per-token cost
         est = sum(by_name[k]["ms_per_launch_events"] for k in own if k in by_name)
