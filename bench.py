@@ -190,7 +190,7 @@ def make_workloads(torch, lib, stream_handle, rotate):
         lens = torch.randint(256, 513, (batch,), generator=g, dtype=torch.int32)
         tokens = int(lens.sum())
         w.name, w.dtype, w.tokens = "qkv_bias_rope_transpose_%s_b8_s512" % sfx, sfx, tokens
-        w.kernel = "isp::qkv_rope_wave<%s, 128, 2, 4>" % ("__half" if es == 2 else "float")
+        w.kernel = "isp::qkv_rope_lean_f16<2, true>" if es == 2 else "isp::qkv_rope_wave<float, 128, 2, 4>"
         w.bytes_per_launch = tokens * (2 * (hn + 2 * kvn) * hs * es + 4) + (hn + 2 * kvn) * hs * es + 2 * batch * 4
         lens_d = lens.to(dev)
         po = torch.zeros((batch, seq), device=dev, dtype=torch.int32)

@@ -224,7 +224,10 @@ typedef enum isp_tuning_knob {
                                         3 = a workgroup per 4 KiB chunk of a row (default) */
     ISP_TUNE_EMBED_STORE = 5,        /* 1 = plain, 2 = non-temporal, 3 = write-through (default) */
     ISP_TUNE_QKV_STORE = 6,          /* 1 = plain, 2 = non-temporal, 3 = write-through (default) */
-    ISP_TUNE_QKV_WAVES = 7,          /* waves (groups of 8 heads) per workgroup: 1, 2 or 4 (default) */
+    ISP_TUNE_QKV_WAVES = 7,          /* 1, 2 or 4: the general kernel with that many waves (groups of 8 heads) per
+                                        workgroup; 0 = automatic: the fp16 one-vector-per-lane kernel where the shape
+                                        allows it (128-element heads fully rotated, head counts multiples of 32),
+                                        else the general kernel with 4 waves */
     ISP_TUNE_COUNT = 8
 } isp_tuning_knob;
 int isp_tuning_set(int knob, int value);

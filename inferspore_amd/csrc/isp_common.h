@@ -75,10 +75,15 @@ __device__ __forceinline__ void store16_stream(void* p, const vec16& v) {
 // one-instruction asm.  It is a vector-memory store like any other; the only thing the compiler does
 // not see is its entry in the vector-memory counter, which can only make the waits it computes for
 // later loads longer, never shorter (loads complete in order among themselves).
+// The trailing s_nop is part of the instruction's contract on this hardware: a vector-memory store of
+// more than 8 bytes reads its data registers one cycle after issue, and an instruction that rewrites
+// them must not follow directly.  The compiler inserts that wait state for its own stores but cannot
+// see into an asm block (without it, a second store whose address landed in the first store's data
+// registers wrote address bits into the first one's output, a few elements per million).
 __device__ __forceinline__ void store16_through(void* p, const vec16& v) {
     typedef uint32_t u4 __attribute__((ext_vector_type(4)));
     u4 t = {v.w[0], v.w[1], v.w[2], v.w[3]};
-    asm volatile("global_store_dwordx4 %0, %1, off sc1 nt" : : "v"(p), "v"(t) : "memory");
+    asm volatile("global_store_dwordx4 %0, %1, off sc1 nt\n\ts_nop 1" : : "v"(p), "v"(t) : "memory");
 }
 
 // Store kinds selectable per kernel instantiation.

@@ -10,18 +10,20 @@
 //   v heads and un-rotated elements are copied;  destination [b, head, s, :] of q / k / v.
 //
 // Design (not the reference's one-thread-per-element, one-block-per-(token, head) kernel):
-//   * a lane owns 16 bytes at d = VEC*g and the 16 bytes of the rotation partners at d + hs/2, so
-//     the rotate-half pairing needs no cross-lane exchange, and each group of hs/(2 VEC) lanes
-//     reads and writes whole 128-byte lines of one 256-byte head row;
-//   * a wave carries 8 heads (fp16) of one token, a workgroup 32; the 64 distinct (cos, sin) pairs
-//     of the token are evaluated once per workgroup, one pair per lane of its first wave, and
-//     handed to the other waves through 512 bytes of LDS behind a barrier that they reach while
-//     their own loads are in flight (the reference evaluates powf + cos + sin for every (head, d));
-//   * the divisors base^(2d/rot) do not depend on the data, so the host computes them once per
-//     call with the C library's powf and passes them by value in the kernel arguments: the device
-//     forms angle = t / divisor with one correctly rounded division;
-//   * loads are issued before the transcendental work; stores are non-temporal (q, k, v are
-//     consumed by a later kernel, not by this one).
+//   * the divisors base^(2d/rot) do not depend on the data, so the host computes them once with the
+//     C library's powf and passes them by value in the kernel arguments; the device forms
+//     angle = t / divisor with one correctly rounded division and evaluates full-range sincosf;
+//   * the token's 64 distinct (cos, sin) pairs are evaluated once per workgroup, one pair per lane
+//     of its first wave, and handed to the other waves through LDS behind a barrier that they reach
+//     while their own loads are in flight (the reference evaluates powf + cos + sin for every
+//     (head, d): 48 to 96 times more transcendental work);
+//   * the streamed loads are issued before anything that depends on padding_offset / history;
+//   * two kernels share this: qkv_rope_lean_f16 for the common LLaMA shape (one 16-byte vector per
+//     lane, partner exchange by DPP, scalar address arithmetic) and qkv_rope_wave for every other
+//     vectorisable shape and for fp32 (a lane owns 16 bytes at d = VEC*g and the 16 bytes of its
+//     rotation partners at d + hs/2, so the rotate-half pairing needs no cross-lane exchange); both
+//     read and write whole 128-byte lines of the 256-byte head rows and give identical bits;
+//   * stores are non-temporal write-through (q, k, v are consumed by a later kernel).
 #include <math.h>
 
 #include "isp_common.h"
@@ -34,10 +36,12 @@ struct RopeDivisors {
     float div[kMaxHalfRot];
 };
 
-// (cos, sin) of timestep / divisor.  Kept out of line so that the prefill, decode and scalar kernels
-// all execute the very same instruction sequence: a decode step at `step` and a prefill token at
-// history = step - 1 then produce identical bits.
-__device__ __attribute__((noinline)) float2 rope_coefficients(int timestep, float divisor) {
+// (cos, sin) of timestep / divisor: one correctly rounded division and the full-range sincosf, the
+// same two operations in every kernel of this file, so a decode step at `step` and a prefill token at
+// history = step - 1 produce identical bits (tested).  Inlined on purpose: a device function call
+// starts by waiting for all outstanding memory operations, which would put the evaluation behind
+// the arrival of the streamed loads instead of underneath it.
+__device__ __forceinline__ float2 rope_coefficients(int timestep, float divisor) {
     float sn, c;
     sincosf((float)timestep / divisor, &sn, &c);
     return make_float2(c, sn);
@@ -84,6 +88,10 @@ __global__ __launch_bounds__(kWave * WAVES) void qkv_rope_wave(
     const int col = g * VEC;
     const T* src = qkv + ((size_t)token * (size_t)qkv_heads + (live ? h : 0)) * HS;
 
+    // divisor first (see qkv_rope_lean_f16): the coefficients then do not wait for the rows
+    const float my_divisor = tab.div[lane < HALF ? lane : 0];
+    asm volatile("" ::: "memory");
+
     // The source address depends on the token index only, so the streamed loads are issued before
     // the destination (padding_offset -> batch row -> history) is known: the dependent scalar
     // loads then overlap the HBM latency instead of preceding it.
@@ -110,7 +118,7 @@ __global__ __launch_bounds__(kWave * WAVES) void qkv_rope_wave(
         __shared__ float2 cs[HALF];
         if (wave == 0 && lane < HALF) {
             float2 coef = make_float2(1.0f, 0.0f);
-            if (lane < half_rot) coef = rope_coefficients(history_length[b] + s, tab.div[lane]);
+            if (lane < half_rot) coef = rope_coefficients(history_length[b] + s, my_divisor);
             cs[lane] = coef;
         }
         __syncthreads();
@@ -157,6 +165,129 @@ __global__ __launch_bounds__(kWave * WAVES) void qkv_rope_wave(
     }
     store16_sel<ST>(dst + col, Elem<T>::pack(y0));
     store16_sel<ST>(dst + HALF + col, Elem<T>::pack(y1));
+}
+
+// Unsigned division by a launch constant without the integer-divide expansion: q = floor(p / d) from
+// one multiply-high and one correction step (exact for every 32-bit p).
+struct FastDiv {
+    unsigned d, m;  // m = floor(2^32 / d), saturated for d = 1
+    __device__ __forceinline__ void divmod(unsigned p, unsigned& q, unsigned& r) const {
+        q = __umulhi(p, m);
+        r = p - q * d;
+        if (r >= d) {
+            q++;
+            r -= d;
+        }
+    }
+};
+
+static FastDiv make_fastdiv(unsigned d) {
+    FastDiv f;
+    f.d = d;
+    f.m = d <= 1 ? 0xffffffffu : (unsigned)(0x100000000ull / d);
+    return f;
+}
+
+// The common LLaMA shape (fp16, head size 128 fully rotated, q and kv head counts multiples of 32)
+// with as few instructions per wave as the arithmetic allows, because at one 16-byte vector per
+// lane a wave moves only 1 KiB and anything above ~100 vector instructions per wave shows up in
+// the run time.  One vector per lane: 512 threads carry the 32 heads of one group (all q, all k or
+// all v) of one token, every load and store instruction of a wave covers 4 whole head rows.  The
+// rotation partner (d +- 64) is 8 lanes away and comes through a DPP row rotation; (cos, sin) are
+// evaluated once per workgroup by its first wave and stored twice, as (c, -s) for the lower and
+// (c, s) for the upper half of a row, so that both halves run out = c * x + t * partner; row,
+// plane and sequence arithmetic is wave-uniform (scalar).  Same operations per element as
+// rotate_pair(), so the results are bit-identical to the other kernels of this file.  BIAS is a
+// template argument so that each variant has a fixed sequence of loads and the compiler's waits
+// are exact for it.
+template <int ST, bool BIAS>
+__global__ __launch_bounds__(512) void qkv_rope_lean_f16(
+    RopeDivisors tab, __half* q, __half* k, __half* v, const __half* qkv, const __half* bias,
+    const int32_t* __restrict__ padding_offset, const int32_t* __restrict__ history_length,
+    unsigned positions, FastDiv seq, unsigned head_num, unsigned kv_head_num) {
+    // (no __restrict__ on the tensors: the compiler would be free to move their loads across the
+    // ordering barriers below, and it then sinks the streamed load behind the padding lookup)
+    constexpr unsigned ROW_BYTES = 256, GROUP = 32;
+    const unsigned tid = threadIdx.x;
+    const unsigned token = blockIdx.x;
+    const unsigned first = blockIdx.y * GROUP;  // first head of this workgroup's group
+    const unsigned qkv_heads = head_num + 2 * kv_head_num;
+
+    // Vector-memory results return in issue order, so this lane's divisor is requested first and the
+    // loads are kept in their order (divisor, streamed row, bias): the wait in front of the
+    // coefficient evaluation then covers the divisor only.  The divisor table is the first kernel argument;
+    // it is read through a plain global pointer to the argument block, because the compiler
+    // treats argument loads as movable at will and would place this one behind the row's.
+    float my_divisor;
+    {
+        typedef const float __attribute__((address_space(1)))* global_floats;
+        unsigned long long block = (unsigned long long)__builtin_amdgcn_kernarg_segment_ptr();
+        asm volatile("" : "+s"(block));
+        my_divisor = reinterpret_cast<global_floats>(block)[tid & 63u];
+        (void)tab;
+    }
+    asm volatile("" ::: "memory");
+    const char* src = reinterpret_cast<const char*>(qkv) + ((size_t)token * qkv_heads + first) * ROW_BYTES;
+    const vec16 raw = load16_stream(src + tid * 16u);
+    asm volatile("" ::: "memory");
+    vec16 braw;
+    if (BIAS) braw = load16(reinterpret_cast<const char*>(bias) + (size_t)first * ROW_BYTES + tid * 16u);
+    asm volatile("" ::: "memory");  // keeps the loads in front of the lookups below
+
+    const long long p = (long long)token + (long long)padding_offset[token];
+    if (p < 0 || p >= (long long)positions) return;  // workgroup-uniform
+    unsigned b, s;
+    seq.divmod((unsigned)p, b, s);
+
+    __half* plane;
+    unsigned plane_heads, h0;
+    const bool rotates = first < head_num + kv_head_num;
+    if (first < head_num) {
+        plane = q, plane_heads = head_num, h0 = first;
+    } else if (rotates) {
+        plane = k, plane_heads = kv_head_num, h0 = first - head_num;
+    } else {
+        plane = v, plane_heads = kv_head_num, h0 = first - head_num - kv_head_num;
+    }
+    char* dst = reinterpret_cast<char*>(plane) + (((size_t)b * plane_heads + h0) * seq.d + s) * ROW_BYTES;
+    const unsigned lane_offset = (tid >> 4) * (seq.d * ROW_BYTES) + (tid & 15u) * 16u;  // head row, column
+
+    if (!rotates && !BIAS) {  // v heads without bias: a plain move
+        store16_sel<ST>(dst + lane_offset, raw);
+        return;
+    }
+    // the coefficient table first: the first wave evaluates it while every wave's loads are in flight
+    __shared__ float2 cs[2][64];
+    if (rotates) {
+        if (tid < 64) {
+            const float2 coef = rope_coefficients(history_length[b] + (int)s, my_divisor);
+            cs[0][tid] = make_float2(coef.x, -coef.y);
+            cs[1][tid] = coef;
+        }
+        __syncthreads();
+    }
+    float x[8], y[8];
+    Elem<__half>::unpack(raw, x);
+    if (BIAS) {
+        float bv[8];
+        Elem<__half>::unpack(braw, bv);
+#pragma unroll
+        for (int e = 0; e < 8; e++) x[e] += bv[e];
+    }
+    if (rotates) {
+        const unsigned upper = (tid >> 3) & 1u;
+        const unsigned pair = (tid & 7u) * 8u;
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            const float2 t = cs[upper][pair + e];
+            const float other = dpp_mov<0x128>(x[e]);  // row_ror:8: the lane 8 further on / back
+            y[e] = __fmaf_rn(t.x, x[e], t.y * other);
+        }
+    } else {
+#pragma unroll
+        for (int e = 0; e < 8; e++) y[e] = x[e];
+    }
+    store16_sel<ST>(dst + lane_offset, Elem<__half>::pack(y));
 }
 
 // Any (even) head size and any alignment: one workgroup per token, one lane per rotation pair.
@@ -388,7 +519,41 @@ static int qkv_rope(void* q_, void* k_, void* v_, const void* qkv_, const void* 
         else ISP_QKV_LAUNCH_K(HS, 4);                                                              \
     } while (0)
     const int head_groups_max = 65535 * 4;  // grid.y limit, 4 heads per workgroup at least
-    if (vec_ok && head_size == 128 && head_num + 2 * kv_head_num <= head_groups_max) {
+    // lean kernel: fp16, 128-element heads fully rotated, whole groups of 32 q / k / v heads, offsets
+    // inside a group and positions inside the batch in 32 bits; ISP_TUNE_QKV_WAVES = 1, 2, 4 opts out
+    const int waves_knob = tuning(ISP_TUNE_QKV_WAVES);
+    const bool lean_ok = sizeof(T) == 2 && vec_ok && head_size == 128 && rot == 128 &&
+                         head_num % 32 == 0 && kv_head_num % 32 == 0 &&
+                         (head_num + 2 * kv_head_num) / 32 <= 65535 &&
+                         (unsigned long long)seq_len * 256ull * 32ull <= 0xffffffffull &&
+                         (unsigned long long)batch * (unsigned long long)seq_len <= 0x7fffffffull &&
+                         (waves_knob <= 0 || waves_knob >= 8);
+    if (lean_ok) {
+        const dim3 g2((unsigned)token_num, (unsigned)((head_num + 2 * kv_head_num) / 32));
+        const unsigned positions = (unsigned)batch * (unsigned)seq_len;
+        const FastDiv fd = make_fastdiv((unsigned)seq_len);
+        __half* qh = reinterpret_cast<__half*>(q);
+        __half* kh = reinterpret_cast<__half*>(k);
+        __half* vh = reinterpret_cast<__half*>(v);
+        const __half* xh = reinterpret_cast<const __half*>(qkv);
+        const __half* bh = reinterpret_cast<const __half*>(bias);
+#define ISP_QKV_LEAN(K)                                                                            \
+    do {                                                                                           \
+        if (bh)                                                                                    \
+            hipLaunchKernelGGL((qkv_rope_lean_f16<K, true>), g2, dim3(512), 0, s, tab, qh, kh, vh,  \
+                               xh, bh, padding_offset, history_length, positions, fd,              \
+                               (unsigned)head_num, (unsigned)kv_head_num);                         \
+        else                                                                                       \
+            hipLaunchKernelGGL((qkv_rope_lean_f16<K, false>), g2, dim3(512), 0, s, tab, qh, kh, vh, \
+                               xh, bh, padding_offset, history_length, positions, fd,              \
+                               (unsigned)head_num, (unsigned)kv_head_num);                         \
+    } while (0)
+        if (kind == kStoreThrough) ISP_QKV_LEAN(kStoreThrough);
+        else if (kind == kStoreStream) ISP_QKV_LEAN(kStoreStream);
+        else ISP_QKV_LEAN(kStorePlain);
+#undef ISP_QKV_LEAN
+        e = hipGetLastError();
+    } else if (vec_ok && head_size == 128 && head_num + 2 * kv_head_num <= head_groups_max) {
         ISP_QKV_LAUNCH_WAVE(128);
         e = hipGetLastError();
     } else if (vec_ok && head_size == 64 && head_num + 2 * kv_head_num <= head_groups_max) {

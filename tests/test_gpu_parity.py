@@ -362,6 +362,30 @@ def test_knobs_do_not_change_results(isp):
             say("qkv knobs %s store=%d waves=%d" % (dtype.__name__, store, waves))
             got = _with_knobs({capi.TUNE_QKV_STORE: store, capi.TUNE_QKV_WAVES: waves}, run_qkv)
             assert all(np.array_equal(a, b) for a, b in zip(got, base))
+    # qkv at the common LLaMA shape: the automatic choice is the one-vector-per-lane fp16 kernel, the
+    # waves knob forces the general kernel; both must give the same bits, with and without bias
+    for with_bias in (True, False):
+        lens, qkv, bias, po, hist = qkv_inputs(2, 24, 32, 32, 128, np.float16, seed=47, min_len=5, with_bias=with_bias)
+        hist = np.array([3, 1000], np.int32)
+        d_in, d_bias, d_po, d_hist, d_lens = dev(qkv), dev(bias), dev(po), dev(hist), dev(lens)
+        tokens = qkv.shape[0]
+        po_dev = torch.zeros((2, 24), dtype=torch.int32, device="cuda")
+        po_dev.view(-1)[:tokens] = d_po
+
+        def run_llama():
+            outs = [torch.full((2, 32, 24, 128), -3, dtype=torch.float16, device="cuda") for _ in range(3)]
+            isp.add_fused_qkv_bias_transpose_and_rope(outs[0], outs[1], outs[2], d_in, d_bias, po_dev, d_hist, d_lens,
+                                                      128, 10000.0)
+            return [host(o) for o in outs]
+
+        base = run_llama()
+        for store, waves in itertools.product((0, 1, 2, 3), (1, 2, 4)):
+            say("qkv llama-shape knobs bias=%s store=%d waves=%d" % (with_bias, store, waves))
+            got = _with_knobs({capi.TUNE_QKV_STORE: store, capi.TUNE_QKV_WAVES: waves}, run_llama)
+            assert all(np.array_equal(a, b) for a, b in zip(got, base))
+        for store in (1, 2, 3):
+            got = _with_knobs({capi.TUNE_QKV_STORE: store}, run_llama)
+            assert all(np.array_equal(a, b) for a, b in zip(got, base))
     # embedding
     ids, table = embedding_inputs(77, 4096, 300, np.float16, seed=43)
     d_ids, d_table = dev(ids), dev(table)
