@@ -47,6 +47,19 @@ __device__ __forceinline__ float2 rope_coefficients(int timestep, float divisor)
     return make_float2(c, sn);
 }
 
+// Word `index` of the first kernel argument (the divisor table), read through a plain global pointer
+// to the argument block.  Vector-memory results return in issue order; qkv_rope_lean_f16 wants this
+// word requested before its streamed row, so that the coefficient evaluation waits for it alone.
+// An ordinary argument access would not do: the compiler treats argument loads as movable at will
+// and places this one behind the rows'.  The tensors of such a kernel carry no __restrict__ for the
+// same reason (their loads must stay where the ordering barriers put them).
+__device__ __forceinline__ float first_argument_word(unsigned index) {
+    typedef const float __attribute__((address_space(1)))* global_floats;
+    unsigned long long block = (unsigned long long)__builtin_amdgcn_kernarg_segment_ptr();
+    asm volatile("" : "+s"(block));
+    return reinterpret_cast<global_floats>(block)[index];
+}
+
 // One rotation, with the contraction spelled out so that every kernel in this file rounds the same
 // way: y0 = c x0 - s x1, y1 = c x1 + s x0, each as one product plus one fused multiply-add.
 __device__ __forceinline__ void rotate_pair(float c, float sn, float x0, float x1, float& y0,
@@ -88,10 +101,6 @@ __global__ __launch_bounds__(kWave * WAVES) void qkv_rope_wave(
     const int col = g * VEC;
     const T* src = qkv + ((size_t)token * (size_t)qkv_heads + (live ? h : 0)) * HS;
 
-    // divisor first (see qkv_rope_lean_f16): the coefficients then do not wait for the rows
-    const float my_divisor = tab.div[lane < HALF ? lane : 0];
-    asm volatile("" ::: "memory");
-
     // The source address depends on the token index only, so the streamed loads are issued before
     // the destination (padding_offset -> batch row -> history) is known: the dependent scalar
     // loads then overlap the HBM latency instead of preceding it.
@@ -118,7 +127,7 @@ __global__ __launch_bounds__(kWave * WAVES) void qkv_rope_wave(
         __shared__ float2 cs[HALF];
         if (wave == 0 && lane < HALF) {
             float2 coef = make_float2(1.0f, 0.0f);
-            if (lane < half_rot) coef = rope_coefficients(history_length[b] + s, my_divisor);
+            if (lane < half_rot) coef = rope_coefficients(history_length[b] + s, tab.div[lane]);
             cs[lane] = coef;
         }
         __syncthreads();
@@ -205,27 +214,15 @@ __global__ __launch_bounds__(512) void qkv_rope_lean_f16(
     RopeDivisors tab, __half* q, __half* k, __half* v, const __half* qkv, const __half* bias,
     const int32_t* __restrict__ padding_offset, const int32_t* __restrict__ history_length,
     unsigned positions, FastDiv seq, unsigned head_num, unsigned kv_head_num) {
-    // (no __restrict__ on the tensors: the compiler would be free to move their loads across the
-    // ordering barriers below, and it then sinks the streamed load behind the padding lookup)
     constexpr unsigned ROW_BYTES = 256, GROUP = 32;
     const unsigned tid = threadIdx.x;
     const unsigned token = blockIdx.x;
     const unsigned first = blockIdx.y * GROUP;  // first head of this workgroup's group
     const unsigned qkv_heads = head_num + 2 * kv_head_num;
 
-    // Vector-memory results return in issue order, so this lane's divisor is requested first and the
-    // loads are kept in their order (divisor, streamed row, bias): the wait in front of the
-    // coefficient evaluation then covers the divisor only.  The divisor table is the first kernel argument;
-    // it is read through a plain global pointer to the argument block, because the compiler
-    // treats argument loads as movable at will and would place this one behind the row's.
-    float my_divisor;
-    {
-        typedef const float __attribute__((address_space(1)))* global_floats;
-        unsigned long long block = (unsigned long long)__builtin_amdgcn_kernarg_segment_ptr();
-        asm volatile("" : "+s"(block));
-        my_divisor = reinterpret_cast<global_floats>(block)[tid & 63u];
-        (void)tab;
-    }
+    // loads in the order divisor, streamed row, bias, and kept in it (see first_argument_word)
+    const float my_divisor = first_argument_word(tid & 63u);
+    (void)tab;
     asm volatile("" ::: "memory");
     const char* src = reinterpret_cast<const char*>(qkv) + ((size_t)token * qkv_heads + first) * ROW_BYTES;
     const vec16 raw = load16_stream(src + tid * 16u);
