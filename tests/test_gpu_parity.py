@@ -295,6 +295,10 @@ def test_qkv_rope_known_answer(isp):
 @pytest.mark.parametrize("batch,seq,hn,kvn,hs,rot", [
     (3, 12, 4, 4, 128, 128),    # vector path, tiny
     (2, 9, 8, 2, 128, 128),     # GQA
+    (2, 9, 32, 8, 128, 128),    # GQA 32q/8kv: one whole q group, one group holding k, v and dead rows
+    (2, 5, 40, 40, 128, 128),   # 120 heads: groups straddle the q/k and k/v boundaries
+    (1, 7, 64, 8, 128, 128),    # 64q/8kv
+    (2, 6, 33, 3, 128, 128),    # head counts that are multiples of nothing
     (2, 9, 5, 1, 128, 64),      # MQA, partial rotary, head counts that do not fill a wave pass
     (3, 7, 4, 2, 64, 64),       # 64-wide heads
     (2, 6, 3, 3, 16, 16),       # scalar kernel
