@@ -254,12 +254,16 @@ __global__ __launch_bounds__(512) void qkv_rope_lean_f16(
         return;
     }
     // the coefficient table first: the first wave evaluates it while every wave's loads are in flight
-    __shared__ float2 cs[2][64];
+    // Table layout [j][class][2]: class = tid & 15 names a lane's column and half row (16 classes),
+    // j = 0..3 its four 16-byte reads of two (c, t) pairs each; the 16 classes of one j are
+    // contiguous (256 bytes = all 64 banks), so the reads of a wave are conflict-free.
+    __shared__ float2 cs[4][16][2];
     if (rotates) {
         if (tid < 64) {
             const float2 coef = rope_coefficients(history_length[b] + (int)s, my_divisor);
-            cs[0][tid] = make_float2(coef.x, -coef.y);
-            cs[1][tid] = coef;
+            const unsigned g = tid >> 3, e = tid & 7u;  // pair tid = element e of column group g
+            cs[e >> 1][g][e & 1u] = make_float2(coef.x, -coef.y);  // lower half row: c x - s partner
+            cs[e >> 1][g + 8][e & 1u] = coef;                      // upper half row: c x + s partner
         }
         __syncthreads();
     }
@@ -272,11 +276,10 @@ __global__ __launch_bounds__(512) void qkv_rope_lean_f16(
         for (int e = 0; e < 8; e++) x[e] += bv[e];
     }
     if (rotates) {
-        const unsigned upper = (tid >> 3) & 1u;
-        const unsigned pair = (tid & 7u) * 8u;
+        const unsigned cls = tid & 15u;
 #pragma unroll
         for (int e = 0; e < 8; e++) {
-            const float2 t = cs[upper][pair + e];
+            const float2 t = cs[e >> 1][cls][e & 1];
             const float other = dpp_mov<0x128>(x[e]);  // row_ror:8: the lane 8 further on / back
             y[e] = __fmaf_rn(t.x, x[e], t.y * other);
         }
