@@ -60,6 +60,9 @@ def parse():
     ap.add_argument("--only", default=None, help="run a single workload by name")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--warm", action="store_true", help="also report cache-warm (no rotation) rates")
+    ap.add_argument("--copy-curve", action="store_true",
+                    help="instead of the workloads, time the plain copy at 8 MiB .. 1 GiB of traffic per launch "
+                         "(the practical ceiling as a function of launch size) and print it as one JSON line")
     ap.add_argument("--cpu-seconds", type=float, default=20.0, help="budget of the CPU baseline leg")
     return ap.parse_args()
 
@@ -95,6 +98,22 @@ class Workload:
             if rc:
                 raise RuntimeError("%s: C ABI returned %d" % (self.name, rc))
         self.launch = launch
+
+
+def make_copy_workload(torch, lib, stream_handle, nbytes):
+    """Plain copy of nbytes (traffic 2 x nbytes per launch), rotating over > 1 GiB of buffers."""
+    w = Workload()
+    w.name, w.dtype, w.tokens = "calibration_copy_%dMiB_traffic" % (2 * nbytes >> 20), "u8", 0
+    w.kernel = "isp::copy_vec<1>"
+    w.bytes_per_launch = 2 * nbytes
+    R = w.sets_for(2 * nbytes, True)
+    srcs = torch.empty((R, nbytes), device="cuda", dtype=torch.uint8).fill_(7)
+    dsts = torch.empty((R, nbytes), device="cuda", dtype=torch.uint8)
+    w.keep = (srcs, dsts)
+    w.bind(lib.isp_calibration_copy, [(dsts[j].data_ptr(), srcs[j].data_ptr(), nbytes, stream_handle) for j in range(R)])
+    w.reset = lambda: None
+    w.config = {"bytes_copied": nbytes}
+    return w
 
 
 def make_workloads(torch, lib, stream_handle, rotate):
@@ -604,6 +623,26 @@ def main():
             lib.isp_calibration_copy(b_buf.data_ptr(), a_buf.data_ptr(), 64 << 20, handle)
         stream.synchronize()
         del a_buf, b_buf
+
+    if a.copy_curve:
+        points = []
+        for mib in (8, 16, 24, 32, 48, 64, 96, 128, 192, 256, 384, 512, 1024):
+            with torch.cuda.stream(stream):
+                w = make_copy_workload(torch, lib, handle, (mib << 20) // 2)
+            torch.cuda.synchronize()
+            r = measure(torch, w, a.steps, a.warmup, stream)
+            points.append({"traffic_MiB": mib, "us_per_launch": r["ms_per_launch_events"] * 1e3, "GBps": r["GBps"],
+                           "frac_of_hbm_peak": r["frac_of_hbm_peak"]})
+            del w
+        # least-squares line  time = fixed + bytes / rate  over the points
+        xs = [p["traffic_MiB"] * 2.0 ** 20 for p in points]
+        ys = [p["us_per_launch"] for p in points]
+        n = len(xs)
+        mx, my = sum(xs) / n, sum(ys) / n
+        slope = sum((x - mx) * (y - my) for x, y in zip(xs, ys)) / sum((x - mx) ** 2 for x in xs)
+        print(json.dumps({"metric": "plain copy (isp_calibration_copy) vs traffic per launch", "unit": "GB/s",
+                          "points": points, "fit": {"fixed_us": my - slope * mx, "asymptotic_GBps": 1e-3 / slope}}))
+        return
 
     results = run_all(True)
     head = results[0]
