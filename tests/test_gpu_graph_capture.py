@@ -79,3 +79,69 @@ def test_capture_and_replay_matches_eager(isp):
         scratch.add_(1.0)
         isp.rmsnorm(torch.randn((4, 4096), device="cuda").half(), t["gamma"], 1e-5)
         torch.cuda.synchronize()
+
+
+def test_capture_of_the_prefill_kernels(isp):
+    """The prefill-side entry points under capture: the gather, the padding-offset builder, the LLaMA-shape
+    QKV kernel (which reads its divisor table straight out of the kernel-argument block, so the block
+    the graph node holds must serve it on every replay), transpose-out and the fused norm."""
+    print("[case] graph capture of the prefill kernels", flush=True)
+    g = torch.Generator(device="cuda").manual_seed(3)
+    batch, seq, hn, hs, vocab, hidden = 4, 48, 32, 128, 500, 4096
+    lens = torch.tensor([48, 17, 30, 5], dtype=torch.int32, device="cuda")
+    tokens = int(lens.sum())
+    t = {
+        "ids": torch.randint(0, vocab, (tokens,), dtype=torch.int32, device="cuda", generator=g),
+        "table": torch.randn((vocab, hidden), device="cuda", generator=g).half(),
+        "emb": torch.zeros((tokens, hidden), dtype=torch.float16, device="cuda"),
+        "po": torch.zeros((batch, seq), dtype=torch.int32, device="cuda"),
+        "cum": torch.zeros((batch + 1,), dtype=torch.int32, device="cuda"),
+        "hist": torch.tensor([0, 100, 7, 2000], dtype=torch.int32, device="cuda"),
+        "qkv": torch.randn((tokens, 3 * hn, hs), device="cuda", generator=g).half(),
+        "bias": (0.02 * torch.randn((3 * hn * hs,), device="cuda", generator=g)).half(),
+        "q": torch.zeros((batch, hn, seq, hs), dtype=torch.float16, device="cuda"),
+        "k": torch.zeros((batch, hn, seq, hs), dtype=torch.float16, device="cuda"),
+        "v": torch.zeros((batch, hn, seq, hs), dtype=torch.float16, device="cuda"),
+        "packed": torch.zeros((tokens, hn, hs), dtype=torch.float16, device="cuda"),
+        "residual": torch.randn((tokens, hidden), device="cuda", generator=g).half(),
+        "gamma": torch.rand((hidden,), device="cuda", generator=g).half(),
+    }
+
+    def sequence():
+        isp.input_embedding(t["ids"], t["emb"], t["table"])
+        isp.cal_padding_offset(t["po"], t["cum"], lens)
+        isp.add_fused_qkv_bias_transpose_and_rope(t["q"], t["k"], t["v"], t["qkv"], t["bias"], t["po"], t["hist"],
+                                                  lens, 128, 10000.0)
+        isp.transpose_out_remove_padding(t["q"], t["po"], t["packed"])
+        isp.fused_add_bias_residual_rmsnorm(t["residual"], t["emb"], None, t["gamma"], 1e-5)
+
+    initial = _snapshot(t)
+    eager = []
+    for _ in range(2):
+        sequence()
+        torch.cuda.synchronize()
+        eager.append(_snapshot(t))
+    for k, v in initial.items():
+        t[k].copy_(v)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        sequence()
+        for k, v in initial.items():
+            t[k].copy_(v)
+        side.synchronize()
+        graph.capture_begin()
+        sequence()
+        graph.capture_end()
+    torch.cuda.synchronize()
+    for step in range(2):
+        graph.replay()
+        torch.cuda.synchronize()
+        for k, v in eager[step].items():
+            assert torch.equal(t[k], v), "replay %d differs from eager in %s" % (step, k)
+        # a launch of the same kernel with other arguments between the replays
+        other = torch.zeros_like(t["q"])
+        isp.add_fused_qkv_bias_transpose_and_rope(other, other.clone(), other.clone(), t["qkv"], None, t["po"],
+                                                  t["hist"], lens, 128, 500000.0)
+        torch.cuda.synchronize()
