@@ -158,6 +158,22 @@ def test_fused_norm_variants(isp, oracle, dtype, wpr, tokens, hidden):
 
 
 @pytest.mark.parametrize("dtype", [np.float16, np.float32])
+@pytest.mark.parametrize("fused", [True, False])
+@pytest.mark.parametrize("tokens,hidden", [(700, 2048), (1024, 4096), (3000, 4096), (4096, 4096), (9000, 2048),
+                                           (2048, 5120), (1100, 8192), (4100, 5120)])
+def test_fused_norm_launch_heuristic_regimes(isp, oracle, dtype, fused, tokens, hidden):
+    """Row counts either side of what the device holds in one round of waves, where the automatic choice
+    of waves per row changes (streaming rule, single-round rule, few-rows split)."""
+    say("norm regimes %s %s %dx%d" % (dtype.__name__, "fused" if fused else "plain", tokens, hidden))
+    threads = oracle.max_threads()
+    oracle.set_threads(min(threads, 16))
+    try:
+        _check_norm(isp, oracle, dtype, tokens, hidden, fused, False, seed=tokens + hidden + int(fused))
+    finally:
+        oracle.set_threads(1)
+
+
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
 @pytest.mark.parametrize("with_res,with_bias,flags", [(True, False, 0), (False, True, 0), (False, False, 0),
                                                       (True, True, 1), (True, False, 1)])
 def test_fused_norm_optional_operands(isp, oracle, dtype, with_res, with_bias, flags):
