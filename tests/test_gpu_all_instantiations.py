@@ -1,0 +1,126 @@
+"""Every compiled kernel instantiation is launched at least once and gives the bits of the default one.
+
+The launchers pick among template instantiations (vectors per lane x waves per row x store kind for the
+norm, head size x store kind x waves for QKV, unroll x store kind for SwiGLU ...).  The parity tests
+pin the defaults against the oracle; this file walks the tuning knobs over shapes chosen so that every
+remaining instantiation runs, and requires bit-identical results (the knobs may change speed only;
+the one exception is the norm's waves per row, which fixes the order of the row sum: each row split is
+checked against the oracle instead).
+"""
+import itertools
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import assert_f16_close, assert_f32_close, norm_inputs, qkv_inputs, swiglu_inputs
+
+pytestmark = pytest.mark.gpu
+NP2T = {np.float16: torch.float16, np.float32: torch.float32}
+
+
+def say(msg):
+    print("[case] " + msg, flush=True)
+
+
+def dev(a):
+    return None if a is None else torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def with_knobs(settings, fn):
+    from inferspore_amd import capi
+    lib = capi.lib()
+    try:
+        for knob, value in settings.items():
+            assert lib.isp_tuning_set(knob, value) >= 0
+        return fn()
+    finally:
+        for knob in settings:
+            lib.isp_tuning_set(knob, 0)
+
+
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+def test_norm_every_vectors_per_lane_waves_per_row_and_store_kind(isp, oracle, dtype):
+    from inferspore_amd import capi
+    vec = 8 if dtype == np.float16 else 4
+    for wpr, nv in itertools.product((1, 2, 4, 8, 16), (1, 2, 4, 8)):
+        hidden = vec * 64 * wpr * nv - (vec if nv > 1 else 0)  # just inside nv vectors per lane, ragged last vector
+        tokens = 5
+        res, out, bias, gamma = norm_inputs(tokens, hidden, dtype, seed=wpr * 10 + nv)
+        d_bias, d_gamma = dev(bias), dev(gamma)
+
+        def run():
+            d_res, d_out = dev(res), dev(out)
+            isp.fused_add_bias_residual_rmsnorm(d_res, d_out, d_bias, d_gamma, 1e-5)
+            return d_res.cpu().numpy(), d_out.cpu().numpy()
+
+        # the order of the row sum depends on the waves per row, so each row split is checked against the
+        # oracle on its own; the store kind cannot change a bit
+        base = with_knobs({capi.TUNE_NORM_WAVES_PER_ROW: wpr}, run)
+        e_res, e_out = oracle.fused_norm(res, out, bias, gamma, 1e-5)
+        assert np.array_equal(base[0], e_res)
+        if dtype == np.float32:
+            assert_f32_close(base[1], e_out, "norm hidden %d" % hidden)
+        else:
+            assert_f16_close(base[1], e_out, "norm hidden %d" % hidden, max_mismatch_fraction=0.05)
+        for store in (1, 2, 3):
+            say("norm %s hidden=%d waves/row=%d vectors/lane=%d store=%d" % (dtype.__name__, hidden, wpr, nv, store))
+            got = with_knobs({capi.TUNE_NORM_WAVES_PER_ROW: wpr, capi.TUNE_NORM_STORE: store}, run)
+            assert np.array_equal(got[0], base[0]) and np.array_equal(got[1], base[1])
+
+
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+@pytest.mark.parametrize("hs", [64, 128])
+def test_qkv_every_head_size_store_kind_and_wave_count(isp, dtype, hs):
+    from inferspore_amd import capi
+    batch, seq, hn, kvn = 3, 16, 12, 4
+    lens, qkv, bias, po, hist = qkv_inputs(batch, seq, hn, kvn, hs, dtype, seed=hs, min_len=2)
+    hist = np.array([0, 9, 300], np.int32)
+    d_in, d_bias, d_hist, d_lens = dev(qkv), dev(bias), dev(hist), dev(lens)
+    po_dev = torch.zeros((batch, seq), dtype=torch.int32, device="cuda")
+    po_dev.view(-1)[:qkv.shape[0]] = dev(po)
+
+    def run():
+        outs = [torch.full((batch, n, seq, hs), -3, dtype=NP2T[dtype], device="cuda") for n in (hn, kvn, kvn)]
+        isp.add_fused_qkv_bias_transpose_and_rope(outs[0], outs[1], outs[2], d_in, d_bias, po_dev, d_hist, d_lens,
+                                                  hs, 10000.0)
+        return [o.cpu().numpy() for o in outs]
+
+    base = run()
+    for store, waves in itertools.product((1, 2, 3), (1, 2, 4)):
+        say("qkv %s hs=%d store=%d waves=%d" % (dtype.__name__, hs, store, waves))
+        got = with_knobs({capi.TUNE_QKV_STORE: store, capi.TUNE_QKV_WAVES: waves}, run)
+        assert all(np.array_equal(a, b) for a, b in zip(got, base))
+
+
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+def test_swiglu_every_unroll_and_store_kind(isp, oracle, dtype):
+    from inferspore_amd import capi
+    x = swiglu_inputs(21, 11008, dtype, seed=5)
+    d_x = dev(x)
+
+    def run():
+        out = torch.zeros((21, 11008), dtype=NP2T[dtype], device="cuda")
+        isp.act(d_x, out)
+        return out.cpu().numpy()
+
+    base = run()
+    if dtype == np.float32:
+        assert_f32_close(base, oracle.swiglu(x), "swiglu")
+    else:
+        assert_f16_close(base, oracle.swiglu(x), "swiglu")
+    for unroll, store in itertools.product((1, 2, 4), (1, 2, 3)):
+        say("swiglu %s unroll=%d store=%d" % (dtype.__name__, unroll, store))
+        assert np.array_equal(with_knobs({capi.TUNE_SWIGLU_UNROLL: unroll, capi.TUNE_SWIGLU_STORE: store}, run), base)
+
+
+def test_calibration_copy(isp):
+    from inferspore_amd import capi
+    lib = capi.lib()
+    st = torch.cuda.current_stream().cuda_stream
+    for nbytes in (16, 4096, (1 << 20) + 16, 48 << 20):
+        say("calibration copy of %d bytes" % nbytes)
+        src = torch.randint(0, 256, (nbytes,), dtype=torch.uint8, device="cuda")
+        dst = torch.zeros(nbytes + 16, dtype=torch.uint8, device="cuda")
+        capi.check(lib.isp_calibration_copy(dst.data_ptr(), src.data_ptr(), nbytes, st), "isp_calibration_copy")
+        assert torch.equal(dst[:nbytes], src) and int(dst[nbytes:].sum()) == 0
