@@ -210,10 +210,7 @@ int isp_repeat_kv_cache_f16(const void* k_cache, const void* v_cache, void* k_ds
  *   copy bandwidth the machine actually reaches.
  * isp_tuning_set: overrides a launch heuristic process-wide (0 restores the automatic choice) and
  *   returns the previous value, or ISP_ERR_BAD_SHAPE for an unknown knob.  For benchmark sweeps;
- *   results do not depend on the knobs, only speed does -- with one exception: the number of waves
- *   per row of the norm kernels fixes the order in which a row's squares are summed, so different
- *   values (and the automatic choice at different token counts) can differ in the last bit of the
- *   normalised output.  For a given shape the result is always the same.
+ *   results never depend on the knobs, only speed does.
  */
 int isp_calibration_copy(void* dst, const void* src, size_t bytes, isp_stream_t stream);
 

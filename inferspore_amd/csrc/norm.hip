@@ -6,7 +6,7 @@
 // registers between the sum of squares and the scaling, so every tensor crosses HBM exactly once
 // (the reference re-reads and read-modify-writes decoder_out); all global accesses are 16-byte
 // vectors; the row sum is a DPP wave reduction plus, when a row spans several waves, one small LDS
-// combine behind a single barrier.
+// combine behind a single barrier, associated the same way under every launch configuration.
 #include "isp_common.h"
 
 namespace isp {
@@ -16,6 +16,16 @@ namespace isp {
 // the row, strided by ROW_THREADS so that every load instruction of a wave covers 1 KiB of
 // contiguous memory.  ST is the store kind of the two outputs (non-temporal by default).
 constexpr int norm_block(int wpr) { return kWave * wpr > kBlock ? kWave * wpr : kBlock; }
+
+// p[0] + ... + p[N-1] as a balanced binary tree, neighbours first; N a power of two.
+template <int N>
+__device__ __forceinline__ float tree_sum(const float* p) {
+    if constexpr (N == 1) {
+        return p[0];
+    } else {
+        return tree_sum<N / 2>(p) + tree_sum<N / 2>(p + N / 2);
+    }
+}
 
 template <typename T, int NV, int WPR, int ST>
 __global__ __launch_bounds__(norm_block(WPR)) void fused_norm_rows(T* __restrict__ residual,
@@ -55,9 +65,10 @@ __global__ __launch_bounds__(norm_block(WPR)) void fused_norm_rows(T* __restrict
     // (measured: 13.3 us instead of 11.7 us at 2048 x 4096 fp16).  bias is loaded where it is used,
     // gamma once the row has been summed (below).
     float x[NV][VEC];
-    float acc = 0.0f;
+    float part[NV];  // sum of squares of each of this lane's vectors
 #pragma unroll
     for (int j = 0; j < NV; j++) {
+        part[j] = 0.0f;
         if (ok[j]) {
             const int vi = lane + j * ROW_THREADS;
             Elem<T>::unpack(vo[j], x[j]);
@@ -78,7 +89,7 @@ __global__ __launch_bounds__(norm_block(WPR)) void fused_norm_rows(T* __restrict
             if (rsd_row && !(flags & ISP_NORM_RESIDUAL_EXCLUDES_BIAS))
                 store16_sel<ST>(rsd_row + (size_t)vi * VEC, Elem<T>::pack(x[j]));
 #pragma unroll
-            for (int e = 0; e < VEC; e++) acc += x[j][e] * x[j][e];
+            for (int e = 0; e < VEC; e++) part[j] += x[j][e] * x[j][e];
         }
     }
 
@@ -90,16 +101,25 @@ __global__ __launch_bounds__(norm_block(WPR)) void fused_norm_rows(T* __restrict
         if (ok[j]) vg[j] = load16(gamma + (size_t)(lane + j * ROW_THREADS) * VEC);
     }
 
-    float total = wave_sum(acc);
-    if (WPR > 1) {
-        __shared__ float partial[BLOCK / kWave];
-        const int wave = threadIdx.x / kWave;
-        if ((threadIdx.x % kWave) == 0) partial[wave] = total;
-        __syncthreads();
-        total = 0.0f;
+    // The row sum is the balanced binary tree over the vector index, lowest bit first: lanes of a wave
+    // (index bits 0-5, wave_sum), then the waves of the row (next bits), then this lane's own vectors
+    // (top bits); absent vectors add exact zeros.  That tree is the same however the row is split
+    // over waves and vectors per lane, so the result does not depend on the launch configuration --
+    // a row gives the same bits in a batch of 1 and in a batch of 16384.
 #pragma unroll
-        for (int w = 0; w < WPR; w++) total += partial[slot * WPR + w];
+    for (int j = 0; j < NV; j++) part[j] = wave_sum(part[j]);
+    if (WPR > 1) {
+        __shared__ float partial[NV][BLOCK / kWave];
+        const int wave = threadIdx.x / kWave;
+        if ((threadIdx.x % kWave) == 0) {
+#pragma unroll
+            for (int j = 0; j < NV; j++) partial[j][wave] = part[j];
+        }
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < NV; j++) part[j] = tree_sum<WPR>(&partial[j][slot * WPR]);
     }
+    const float total = tree_sum<NV>(part);
     const float inv = rsqrtf(total / (float)hidden + eps);
 
 #pragma unroll

@@ -3,9 +3,7 @@
 The launchers pick among template instantiations (vectors per lane x waves per row x store kind for the
 norm, head size x store kind x waves for QKV, unroll x store kind for SwiGLU ...).  The parity tests
 pin the defaults against the oracle; this file walks the tuning knobs over shapes chosen so that every
-remaining instantiation runs, and requires bit-identical results (the knobs may change speed only;
-the one exception is the norm's waves per row, which fixes the order of the row sum: each row split is
-checked against the oracle instead).
+remaining instantiation runs, and requires bit-identical results (the knobs may change speed only).
 """
 import itertools
 
@@ -54,19 +52,40 @@ def test_norm_every_vectors_per_lane_waves_per_row_and_store_kind(isp, oracle, d
             isp.fused_add_bias_residual_rmsnorm(d_res, d_out, d_bias, d_gamma, 1e-5)
             return d_res.cpu().numpy(), d_out.cpu().numpy()
 
-        # the order of the row sum depends on the waves per row, so each row split is checked against the
-        # oracle on its own; the store kind cannot change a bit
-        base = with_knobs({capi.TUNE_NORM_WAVES_PER_ROW: wpr}, run)
+        base = run()
         e_res, e_out = oracle.fused_norm(res, out, bias, gamma, 1e-5)
         assert np.array_equal(base[0], e_res)
         if dtype == np.float32:
             assert_f32_close(base[1], e_out, "norm hidden %d" % hidden)
         else:
             assert_f16_close(base[1], e_out, "norm hidden %d" % hidden, max_mismatch_fraction=0.05)
-        for store in (1, 2, 3):
-            say("norm %s hidden=%d waves/row=%d vectors/lane=%d store=%d" % (dtype.__name__, hidden, wpr, nv, store))
-            got = with_knobs({capi.TUNE_NORM_WAVES_PER_ROW: wpr, capi.TUNE_NORM_STORE: store}, run)
+        # the row sum is one fixed tree whatever the split of the row over waves and vectors per lane
+        for split, store in itertools.product((1, 2, 4, 8, 16), (1, 2, 3)):
+            say("norm %s hidden=%d waves/row=%d store=%d" % (dtype.__name__, hidden, split, store))
+            got = with_knobs({capi.TUNE_NORM_WAVES_PER_ROW: split, capi.TUNE_NORM_STORE: store}, run)
             assert np.array_equal(got[0], base[0]) and np.array_equal(got[1], base[1])
+
+
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+def test_norm_rows_do_not_depend_on_the_batch_they_are_in(isp, dtype):
+    """The launch configuration changes with the number of rows; a row's result must not."""
+    hidden = 4096
+    g = torch.Generator(device="cuda").manual_seed(11)
+    big_out = torch.randn((9000, hidden), device="cuda", generator=g).to(NP2T[dtype])
+    big_res = torch.randn((9000, hidden), device="cuda", generator=g).to(NP2T[dtype])
+    gamma = (0.5 + torch.rand(hidden, device="cuda", generator=g)).to(NP2T[dtype])
+    ref_out, ref_res = big_out.clone(), big_res.clone()
+    isp.fused_add_bias_residual_rmsnorm(ref_res, ref_out, None, gamma, 1e-5)
+    ref_plain = big_out.clone()
+    isp.rmsnorm(ref_plain, gamma, 1e-5)
+    for rows in (1, 3, 64, 700, 2048, 4097):
+        say("norm %s: first %d of 9000 rows alone" % (dtype, rows))
+        o, r = big_out[:rows].clone(), big_res[:rows].clone()
+        isp.fused_add_bias_residual_rmsnorm(r, o, None, gamma, 1e-5)
+        assert torch.equal(o, ref_out[:rows]) and torch.equal(r, ref_res[:rows])
+        o = big_out[:rows].clone()
+        isp.rmsnorm(o, gamma, 1e-5)
+        assert torch.equal(o, ref_plain[:rows])
 
 
 @pytest.mark.parametrize("dtype", [np.float16, np.float32])
