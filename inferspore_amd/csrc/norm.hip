@@ -91,9 +91,10 @@ __global__ __launch_bounds__(norm_block(WPR)) void fused_norm_rows(T* __restrict
 #pragma unroll
             for (int e = 0; e < VEC; e++) part[j] += x[j][e] * x[j][e];
         }
-        // reduced over the wave here, not after the loop: the vectors arrive in order, and the
-        // reduction of this one then runs while the next is still on its way
-        part[j] = wave_sum(part[j]);
+        // With two vectors per lane the first is reduced over the wave here, not after the loop: the
+        // vectors arrive in order, and its reduction then runs while the second is still on its
+        // way (with four or more, waiting for them one by one costs more than it hides).
+        if (NV <= 2) part[j] = wave_sum(part[j]);
     }
 
     // gamma is requested once this lane's part of the row has arrived and been summed: the L2 round
@@ -109,6 +110,10 @@ __global__ __launch_bounds__(norm_block(WPR)) void fused_norm_rows(T* __restrict
     // (top bits); absent vectors add exact zeros.  That tree is the same however the row is split
     // over waves and vectors per lane, so the result does not depend on the launch configuration --
     // a row gives the same bits in a batch of 1 and in a batch of 16384.
+    if (NV > 2) {
+#pragma unroll
+        for (int j = 0; j < NV; j++) part[j] = wave_sum(part[j]);
+    }
     if (WPR > 1) {
         __shared__ float partial[NV][BLOCK / kWave];
         const int wave = threadIdx.x / kWave;
