@@ -32,20 +32,20 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published peak
 # scaled by what the same counter reads for isp_calibration_copy of known size: x1.9988 and x1.0000).
 # The summary of those runs is profiles/all_kernels_benchmark_shapes.hbm_traffic_pmc.txt.
 MEASURED_TRAFFIC_BYTES = {
-    "fused_add_bias_residual_rmsnorm_f16_2048x4096": 67270562,
+    "fused_add_bias_residual_rmsnorm_f16_2048x4096": 67273632,
     "rmsnorm_f32_64x4096": 2259266,
-    "rmsnorm_f32_16384x4096": 536986872,
-    "embedding_f16_8192x4096_v32000": 133199311,
-    "qkv_bias_rope_transpose_f16_b8_s512": 146722532,
-    "swiglu_f16_prefill_8192x11008": 540885737,
+    "rmsnorm_f32_16384x4096": 536927351,
+    "embedding_f16_8192x4096_v32000": 133201229,
+    "qkv_bias_rope_transpose_f16_b8_s512": 146722659,
+    "swiglu_f16_prefill_8192x11008": 540885097,
     "swiglu_f16_decode_256x11008": 16930411,
     "transpose_remove_padding_f16_b8_s512": 48991558,
     "concat_kv_cache_f16_b8_q512_S1024": 97552773,
     "repeat_kv_cache_f16_b8_k512_S1024": 97552773,
     "rope_decode_f16_1x96x128": 45295,
-    "fused_add_bias_residual_rmsnorm_f32_2048x4096": 134500834,
-    "embedding_f32_8192x4096_v32000": 265216458,
-    "qkv_bias_rope_transpose_f32_b8_s512": 293213134,
+    "fused_add_bias_residual_rmsnorm_f32_2048x4096": 134509277,
+    "embedding_f32_8192x4096_v32000": 265235647,
+    "qkv_bias_rope_transpose_f32_b8_s512": 293212366,
     "swiglu_f32_prefill_8192x11008": 1081746143,
     "calibration_copy_64MiB_traffic": 67108864,
     "calibration_copy_512MiB_traffic": 536734799,
