@@ -1,55 +1,40 @@
 #!/usr/bin/env python3
 """Benchmark of the fused per-layer kernels on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only NAME] [--no-cpu] [--warm]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only NAME] [--no-cpu] [--warm] [--full]
 
 Prints ONE JSON line.  The headline workload is the fused add-bias + residual + RMSNorm in fp16 at
-2048 tokens x 4096 hidden (one step = one launch over one batch); `kernels` carries the same
-measurement for every kernel of the path at its LLaMA-2-7B shape.
+2048 tokens x 4096 hidden (one step = one launch over one batch); `roofline.per_config` carries the
+same measurement for every kernel of the path at its LLaMA-2-7B shape.
 
 Method
-  * inputs are synthetic (torch RNG on the device), resident in HBM before the timed region;
+  * inputs are synthetic (torch's seeded device RNG), resident in HBM before the timed region;
   * every launch works on the next of R buffer sets, R chosen so the sets together exceed 1 GiB:
     successive launches cannot be served from the 256 MB last-level cache ("cold"; --warm disables
     the rotation and is reported separately, never as `value`);
-  * K launches are issued back to back on a private stream between two HIP events recorded on that
-    stream, bracketed by synchronize on both sides; ms_per_step is the host wall clock over the
-    same region, roofline.achieved uses the event time / K (so it includes the gaps between
-    consecutive launches and is a lower bound on the in-kernel rate);
-  * achieved = algorithmic bytes per launch (each operand once: compulsory reads + writes) / time.
+  * after W warm-up launches and a synchronize, a few untimed lead-in launches keep the queue busy and
+    then several regions of exactly K launches each are issued back to back on a private stream, with a
+    HIP event recorded on that stream at every region boundary; the reported time per launch is the
+    MEDIAN region's event time / K (it includes the gaps between consecutive launches and the cost of
+    the event markers, so it is a lower bound on the in-kernel rate); ms_per_step is the host wall
+    clock over all regions / launches, bracketed by synchronize on both sides;
+  * achieved = algorithmic bytes per launch (each operand once: compulsory reads + writes) / time;
+  * roofline.traffic = HBM bytes per launch from rocprofv3 counters, read from
+    profiles/hbm_traffic_per_launch.json (written by `python -m inferspore_amd.profile_summary`);
   * cpu_baseline: the C oracle (a port of the reference's CPU test functions) timed on the host
-    cores of the same machine, on the same workload shape, single thread plus an OpenMP run.
+    cores of the same machine, on the same workload shapes, single thread plus an OpenMP run.
 """
 import argparse
+import ctypes
 import json
 import os
 import sys
 import time
 
+ROOT = os.path.dirname(os.path.abspath(__file__))
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published peak
-
-# HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE and WRITE_SIZE in separate runs, each
-# scaled by what the same counter reads for isp_calibration_copy of known size: x1.9988 and x1.0000).
-# The summary of those runs is profiles/all_kernels_benchmark_shapes.hbm_traffic_pmc.txt.
-MEASURED_TRAFFIC_BYTES = {
-    "fused_add_bias_residual_rmsnorm_f16_2048x4096": 67273632,
-    "rmsnorm_f32_64x4096": 2259266,
-    "rmsnorm_f32_16384x4096": 536927351,
-    "embedding_f16_8192x4096_v32000": 133201229,
-    "qkv_bias_rope_transpose_f16_b8_s512": 146722659,
-    "swiglu_f16_prefill_8192x11008": 540885097,
-    "swiglu_f16_decode_256x11008": 16930411,
-    "transpose_remove_padding_f16_b8_s512": 48991558,
-    "concat_kv_cache_f16_b8_q512_S1024": 97552773,
-    "repeat_kv_cache_f16_b8_k512_S1024": 97552773,
-    "rope_decode_f16_1x96x128": 45295,
-    "fused_add_bias_residual_rmsnorm_f32_2048x4096": 134509277,
-    "embedding_f32_8192x4096_v32000": 265235647,
-    "qkv_bias_rope_transpose_f32_b8_s512": 293212366,
-    "swiglu_f32_prefill_8192x11008": 1081746143,
-    "calibration_copy_64MiB_traffic": 67108864,
-    "calibration_copy_512MiB_traffic": 536734799,
-}
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic_per_launch.json")
+HEADLINE = "fused_add_bias_residual_rmsnorm_f16_2048x4096"
 
 
 def parse():
@@ -57,15 +42,30 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--regions", type=int, default=0,
+                    help="timed regions of --steps launches per workload (default: enough for 300 launches, at least 5)")
     ap.add_argument("--only", default=None, help="run a single workload by name")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--kernels-only", action="store_true",
+                    help="only the per-kernel workloads (no layer, decode-sequence, warm-cache or CPU legs) and a "
+                         "`dispatch_log` of every launch in order: the form profile runs use")
     ap.add_argument("--warm", action="store_true",
                     help="report cache-warm (no rotation) rates for every workload, not only the hot-path ones")
+    ap.add_argument("--full", action="store_true", help="also print the verbose per-workload records (`kernels`)")
     ap.add_argument("--copy-curve", action="store_true",
                     help="instead of the workloads, time the plain copy at 8 MiB .. 1 GiB of traffic per launch "
                          "(the practical ceiling as a function of launch size) and print it as one JSON line")
     ap.add_argument("--cpu-seconds", type=float, default=20.0, help="budget of the CPU baseline leg")
     return ap.parse_args()
+
+
+def measured_traffic():
+    """HBM bytes per launch per workload, as the last committed profile run measured them."""
+    try:
+        with open(TRAFFIC_FILE) as f:
+            return json.load(f).get("bytes_per_launch", {})
+    except (OSError, ValueError):
+        return {}
 
 
 # --------------------------------------------------------------------------- workloads
@@ -83,6 +83,7 @@ class Workload:
     kernel = ""
     sets = 1
     keep = None
+    launches_per_step = 1
 
     @staticmethod
     def sets_for(set_bytes, rotate):
@@ -100,14 +101,35 @@ class Workload:
                 raise RuntimeError("%s: C ABI returned %d" % (self.name, rc))
         self.launch = launch
 
+    def bind_pair(self, fn_a, args_a, fn_b, args_b):
+        """Two dependent launches per step (a fused kernel's unfused counterpart)."""
+        n = len(args_a)
+        self.sets = n
+        self.launches_per_step = 2
 
-def make_copy_workload(torch, lib, stream_handle, nbytes):
+        def launch(i):
+            rc = fn_a(*args_a[i % n]) or fn_b(*args_b[i % n])
+            if rc:
+                raise RuntimeError("%s: C ABI returned %d" % (self.name, rc))
+        self.launch = launch
+
+
+def norm_kernel_name(lib, es, tokens, hidden, fused):
+    v = [ctypes.c_int() for _ in range(4)]
+    rc = lib.isp_norm_launch_config(es, tokens, hidden, int(fused), *[ctypes.byref(x) for x in v])
+    if rc:
+        return "isp::fused_norm_generic"
+    return "isp::fused_norm_rows<%s, %d, %d, %d, %d>" % ("__half" if es == 2 else "float", v[1].value, v[0].value,
+                                                          v[3].value, v[2].value)
+
+
+def make_copy_workload(torch, lib, stream_handle, nbytes, rotate=True):
     """Plain copy of nbytes (traffic 2 x nbytes per launch), rotating over > 1 GiB of buffers."""
     w = Workload()
     w.name, w.dtype, w.tokens = "calibration_copy_%dMiB_traffic" % (2 * nbytes >> 20), "u8", 0
     w.kernel = "isp::copy_vec<1>"
     w.bytes_per_launch = 2 * nbytes
-    R = w.sets_for(2 * nbytes, True)
+    R = w.sets_for(2 * nbytes, rotate)
     srcs = torch.empty((R, nbytes), device="cuda", dtype=torch.uint8).fill_(7)
     dsts = torch.empty((R, nbytes), device="cuda", dtype=torch.uint8)
     w.keep = (srcs, dsts)
@@ -140,28 +162,7 @@ def make_workloads(torch, lib, stream_handle, rotate):
         bias = (0.02 * torch.randn(hidden, device=dev)).to(tdtype) if fused else None
         gamma = (0.5 + torch.rand(hidden, device=dev)).to(tdtype)
         w.keep = (outs, ress, bias, gamma)
-        # the instantiation the launch heuristic picks for this shape (vectors per lane, waves per row)
-        nvec = hidden // (16 // es)
-        vpl = lambda w_: -(-nvec // (64 * w_))
-        want = nvec * (2 if fused else 1)
-        wpr = 1
-        while wpr < 16 and 3 * 64 * wpr < want:
-            wpr *= 2
-        capacity = 32 * torch.cuda.get_device_properties(0).multi_processor_count
-        if tokens * wpr > capacity:
-            w_ = wpr // 2
-            while w_ >= 1:
-                if tokens * w_ <= capacity:
-                    if vpl(w_) <= 4:
-                        wpr = w_
-                    break
-                w_ //= 2
-        else:
-            while wpr < 16 and vpl(wpr) > 1 and tokens * wpr < capacity // 2:
-                wpr *= 2
-        nv = vpl(wpr)
-        nv = 1 if nv <= 1 else 2 if nv <= 2 else 4 if nv <= 4 else 8
-        w.kernel = "isp::fused_norm_rows<%s, %d, %d, 1>" % ("__half" if es == 2 else "float", nv, wpr)
+        w.kernel = norm_kernel_name(lib, es, tokens, hidden, fused)
         if fused:
             fn = getattr(lib, "isp_fused_add_bias_residual_rmsnorm_" + sfx)
             w.bind(fn, [(ress[j].data_ptr(), outs[j].data_ptr(), bias.data_ptr(), gamma.data_ptr(), 1e-5, tokens,
@@ -201,36 +202,41 @@ def make_workloads(torch, lib, stream_handle, rotate):
         w.config = {"tokens": tokens, "hidden": hidden, "vocab": vocab}
         return w
 
-    def qkv(tdtype=torch.float16):
-        w = Workload()
-        es = 2 if tdtype == torch.float16 else 4
-        sfx = "f16" if es == 2 else "f32"
-        batch, seq, hn, kvn, hs = 8, 512, 32, 32, 128
-        g = torch.Generator(device="cpu").manual_seed(0)
-        lens = torch.randint(256, 513, (batch,), generator=g, dtype=torch.int32)
-        tokens = int(lens.sum())
-        w.name, w.dtype, w.tokens = "qkv_bias_rope_transpose_%s_b8_s512" % sfx, sfx, tokens
-        w.kernel = "isp::qkv_rope_lean_f16<2, true>" if es == 2 else "isp::qkv_rope_wave<float, 128, 2, 4>"
-        w.bytes_per_launch = tokens * (2 * (hn + 2 * kvn) * hs * es + 4) + (hn + 2 * kvn) * hs * es + 2 * batch * 4
+    def padded_batch():
+        batch, seq = 8, 512
+        lens = bench_lengths(torch, batch)
         lens_d = lens.to(dev)
         po = torch.zeros((batch, seq), device=dev, dtype=torch.int32)
         cum = torch.zeros((batch + 1,), device=dev, dtype=torch.int32)
-        rc = lib.isp_cal_padding_offset(po.data_ptr(), cum.data_ptr(), lens_d.data_ptr(), batch, seq, st)
-        assert rc == 0
+        assert lib.isp_cal_padding_offset(po.data_ptr(), cum.data_ptr(), lens_d.data_ptr(), batch, seq, st) == 0
+        return batch, seq, int(lens.sum()), lens_d, po
+
+    def qkv(tdtype=torch.float16, hn=32, kvn=32, hs=128, tag=""):
+        w = Workload()
+        es = 2 if tdtype == torch.float16 else 4
+        sfx = "f16" if es == 2 else "f32"
+        batch, seq, tokens, lens_d, po = padded_batch()
+        w.name, w.dtype, w.tokens = "qkv_bias_rope_transpose_%s_b8_s512%s" % (sfx, tag), sfx, tokens
+        if es == 2 and hs == 128 and hn % 32 == 0 and kvn % 32 == 0:
+            w.kernel = "isp::qkv_rope_lean_f16<2, true>"
+        else:
+            w.kernel = "isp::qkv_rope_wave<%s, %d, 2, 4>" % ("__half" if es == 2 else "float", hs)
+        w.bytes_per_launch = tokens * (2 * (hn + 2 * kvn) * hs * es + 4) + (hn + 2 * kvn) * hs * es + 2 * batch * 4
         hist = torch.zeros(batch, device=dev, dtype=torch.int32)
         bias = (0.02 * torch.randn((hn + 2 * kvn) * hs, device=dev)).to(tdtype)
-        set_bytes = tokens * (hn + 2 * kvn) * hs * es + 3 * batch * hn * seq * hs * es
+        set_bytes = tokens * (hn + 2 * kvn) * hs * es + batch * (hn + 2 * kvn) * seq * hs * es
         R = w.sets_for(set_bytes, rotate)
         ins = [torch.randn((tokens, hn + 2 * kvn, hs), device=dev).to(tdtype) for _ in range(R)]
         outs = [[torch.zeros((batch, n, seq, hs), device=dev, dtype=tdtype) for n in (hn, kvn, kvn)]
                 for _ in range(R)]
-        w.keep = (lens_d, po, cum, hist, bias, ins, outs)
+        w.keep = (lens_d, po, hist, bias, ins, outs)
         w.bind(getattr(lib, "isp_qkv_bias_rope_transpose_" + sfx),
                [(outs[j][0].data_ptr(), outs[j][1].data_ptr(), outs[j][2].data_ptr(), ins[j].data_ptr(),
                  bias.data_ptr(), po.data_ptr(), hist.data_ptr(), lens_d.data_ptr(), batch, seq, tokens, hn, kvn, hs,
-                 128, 10000.0, 2048, 0, st) for j in range(R)])
+                 hs, 10000.0, 2048, 0, st) for j in range(R)])
         w.reset = lambda: None
-        w.config = {"batch": batch, "max_seq": seq, "valid_tokens": tokens, "heads": "32q/32kv", "head_dim": hs}
+        w.config = {"batch": batch, "max_seq": seq, "valid_tokens": tokens, "heads": "%dq/%dkv" % (hn, kvn),
+                    "head_dim": hs}
         return w
 
     def swiglu(tokens, tag, tdtype=torch.float16):
@@ -250,16 +256,6 @@ def make_workloads(torch, lib, stream_handle, rotate):
         w.reset = lambda: None
         w.config = {"tokens": tokens, "inter": inter}
         return w
-
-    def padded_batch():
-        batch, seq = 8, 512
-        g = torch.Generator(device="cpu").manual_seed(0)
-        lens = torch.randint(256, 513, (batch,), generator=g, dtype=torch.int32)
-        lens_d = lens.to(dev)
-        po = torch.zeros((batch, seq), device=dev, dtype=torch.int32)
-        cum = torch.zeros((batch + 1,), device=dev, dtype=torch.int32)
-        assert lib.isp_cal_padding_offset(po.data_ptr(), cum.data_ptr(), lens_d.data_ptr(), batch, seq, st) == 0
-        return batch, seq, int(lens.sum()), lens_d, po
 
     def transpose_out():
         w = Workload()
@@ -323,23 +319,10 @@ def make_workloads(torch, lib, stream_handle, rotate):
         return w
 
     def copy(nbytes):
-        # calibration: a plain copy with the same traffic as the headline workload
-        w = Workload()
-        w.name, w.dtype, w.tokens = "calibration_copy_%dMiB_traffic" % (2 * nbytes >> 20), "u8", 0
-        w.kernel = "isp::copy_vec<1>"
-        w.bytes_per_launch = 2 * nbytes
-        R = w.sets_for(2 * nbytes, rotate)
-        srcs = [torch.empty(nbytes, device=dev, dtype=torch.uint8).fill_(j & 255) for j in range(R)]
-        dsts = [torch.empty(nbytes, device=dev, dtype=torch.uint8) for _ in range(R)]
-        w.keep = (srcs, dsts)
-        w.bind(lib.isp_calibration_copy, [(dsts[j].data_ptr(), srcs[j].data_ptr(), nbytes, st) for j in range(R)])
-        w.reset = lambda: None
-        w.config = {"bytes_copied": nbytes}
-        return w
+        return make_copy_workload(torch, lib, st, nbytes, rotate)
 
-    return [
-        ("fused_add_bias_residual_rmsnorm_f16_2048x4096",
-         lambda: norm("fused_add_bias_residual_rmsnorm_f16_2048x4096", 2048, 4096, torch.float16, True)),
+    table = [
+        (HEADLINE, lambda: norm(HEADLINE, 2048, 4096, torch.float16, True)),
         ("rmsnorm_f32_64x4096", lambda: norm("rmsnorm_f32_64x4096", 64, 4096, torch.float32, False)),
         ("rmsnorm_f32_16384x4096", lambda: norm("rmsnorm_f32_16384x4096", 16384, 4096, torch.float32, False)),
         ("embedding_f16_8192x4096_v32000", embedding),
@@ -359,11 +342,24 @@ def make_workloads(torch, lib, stream_handle, rotate):
         ("calibration_copy_64MiB_traffic", lambda: copy(32 << 20)),
         ("calibration_copy_512MiB_traffic", lambda: copy(256 << 20)),
     ]
+    return table
 
 
 # --------------------------------------------------------------------------- timing
 
-def time_workload(torch, w, steps, warmup, stream):
+LEAD_IN = 8   # untimed launches in front of the first region, so that it does not start on an empty queue
+
+
+def region_count(steps, requested):
+    if requested > 0:
+        return requested
+    return max(5, -(-300 // max(steps, 1)))
+
+
+def time_workload(torch, w, steps, warmup, regions, stream):
+    """W warm-up launches, synchronize, then `regions` back-to-back regions of exactly `steps` launches
+    with an event at every boundary.  Returns (wall ms per launch over all regions, median region's
+    event ms per launch, fastest, slowest)."""
     with torch.cuda.stream(stream):
         w.reset()
         for i in range(warmup):
@@ -371,32 +367,38 @@ def time_workload(torch, w, steps, warmup, stream):
         stream.synchronize()
         w.reset()
         torch.cuda.synchronize()
-        e0 = torch.cuda.Event(enable_timing=True)
-        e1 = torch.cuda.Event(enable_timing=True)
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(regions + 1)]
+        n = 0
         t0 = time.perf_counter()
-        e0.record(stream)
-        for i in range(steps):
-            w.launch(i)
-        e1.record(stream)
+        for _ in range(LEAD_IN):
+            w.launch(n)
+            n += 1
+        for r in range(regions):
+            ev[r].record(stream)
+            for _ in range(steps):
+                w.launch(n)
+                n += 1
+        ev[regions].record(stream)
         stream.synchronize()
         torch.cuda.synchronize()
         t1 = time.perf_counter()
-    wall_ms = (t1 - t0) * 1e3 / steps
-    event_ms = e0.elapsed_time(e1) / steps
-    return wall_ms, event_ms
+    per = sorted(ev[r].elapsed_time(ev[r + 1]) / steps for r in range(regions))
+    wall_ms = (t1 - t0) * 1e3 / (regions * steps + LEAD_IN)
+    return wall_ms, per[len(per) // 2], per[0], per[-1]
 
 
-def measure(torch, w, steps, warmup, stream):
-    wall_ms, event_ms = time_workload(torch, w, steps, warmup, stream)
+def measure(torch, w, steps, warmup, regions, stream, traffic):
+    wall_ms, event_ms, fastest, slowest = time_workload(torch, w, steps, warmup, regions, stream)
     gbs = w.bytes_per_launch / (event_ms * 1e-3) / 1e9
     return {
         "workload": w.name, "kernel": w.kernel, "dtype": w.dtype, "tokens": w.tokens, "buffer_sets": w.sets,
-        "algorithmic_bytes": w.bytes_per_launch,
+        "algorithmic_bytes": w.bytes_per_launch, "launches_per_step": w.launches_per_step,
         "ms_per_step_wall": wall_ms, "ms_per_launch_events": event_ms,
+        "ms_fastest_region": fastest, "ms_slowest_region": slowest, "regions": regions,
         "GBps": gbs, "frac_of_hbm_peak": gbs / HBM_PEAK_GBS,
         "tokens_per_s": (w.tokens / (event_ms * 1e-3)) if w.tokens else None,
-        "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": gbs / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC_BYTES.get(w.name)},
+        "traffic": traffic.get(w.name),
+        "launches_total": warmup + LEAD_IN + regions * steps,
     }
 
 
@@ -409,8 +411,7 @@ def context_layer_record(torch, steps, warmup, stream):
     from inferspore_amd.context_layer import BatchState, LayerWeights, context_decoder_layer
     nh, hs, inter, seq, batch = 32, 128, 11008, 512, 8
     hidden = nh * hs
-    g = torch.Generator(device="cpu").manual_seed(0)
-    lens = torch.randint(256, 513, (batch,), generator=g, dtype=torch.int32).tolist()
+    lens = bench_lengths(torch, batch).tolist()
     with torch.cuda.stream(stream):
         w = LayerWeights(hidden, inter, torch.float16)
         st = BatchState(lens, seq, nh, nh, hs, inter, max_seq_len=seq, layers=1, dtype=torch.float16)
@@ -489,12 +490,20 @@ def decode_sequence_record(torch, stream):
 
 # --------------------------------------------------------------------------- CPU baseline
 
-def cpu_baseline(budget_s):
-    """Times the C oracle (a port of the reference's CPU test functions) on the host cores, per kernel,
-    on bounded samples of the benchmark workloads: single thread (as the reference's loops are written)
-    and OpenMP over token rows.  The headline entry is the fused norm at its full size."""
+def bench_lengths(torch, batch=8, lo=256, hi=512):
+    """The ragged batch of the QKV configuration: per-sequence lengths uniform in [256, 512], seed 0."""
+    g = torch.Generator(device="cpu").manual_seed(0)
+    return torch.randint(lo, hi + 1, (batch,), generator=g, dtype=torch.int32)
+
+
+def cpu_baseline(budget_s, lens):
+    """Times the C oracle (a port of the reference's CPU test functions, tests/unittests/*.cu) on the
+    host cores, once per BASELINE configuration at its full size: single thread (as the reference's
+    loops are written) and OpenMP over token rows on every core this job may use.  Where one thread
+    would take too long for the budget it runs a stated sample of the rows.  The headline entry is the
+    fused norm at its full size."""
     import numpy as np
-    sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+    sys.path.insert(0, ROOT)
     from oracle import load
     o = load()
     L = o.lib
@@ -502,9 +511,17 @@ def cpu_baseline(budget_s):
     f16 = np.float16
 
     def normal(*shape, scale=1.0, dtype=f16):
-        return (scale * r.standard_normal(shape, dtype=np.float32)).astype(dtype)
+        a = r.standard_normal(shape, dtype=np.float32)
+        if scale != 1.0:
+            a *= scale
+        return a.astype(dtype)
 
-    samples = []   # (workload, description, tokens, algorithmic bytes, callable, fresh-inputs callable or None)
+    def p(a):
+        return a.ctypes.data
+
+    # (workload, tokens, bytes, full callable, reset or None, one-thread callable or None, one-thread
+    #  tokens, one-thread bytes, sample note, cache note)
+    samples = []
 
     tokens, hidden = 2048, 4096
     out, res = normal(tokens, hidden), normal(tokens, hidden)
@@ -514,38 +531,68 @@ def cpu_baseline(budget_s):
     def norm_reset():
         wa[...] = out
         wb[...] = res
-    samples.append(("fused_add_bias_residual_rmsnorm_f16_2048x4096", "full workload", tokens,
-                    4 * tokens * hidden * 2 + 2 * hidden * 2,
-                    lambda: L.isp_oracle_fused_norm_f16(wb.ctypes.data, wa.ctypes.data, bias.ctypes.data,
-                                                        gamma.ctypes.data, 1e-5, tokens, hidden, 0), norm_reset))
+    nb = 4 * tokens * hidden * 2 + 2 * hidden * 2
+    samples.append(dict(workload=HEADLINE, tokens=tokens, bytes=nb, reset=norm_reset,
+                        fn=lambda: L.isp_oracle_fused_norm_f16(p(wb), p(wa), p(bias), p(gamma), 1e-5, tokens, hidden, 0),
+                        sample="full workload", cache="64 MiB working set: exceeds one core's caches, may sit in a "
+                                                      "large shared L3 between repetitions"))
     x32 = normal(64, hidden, dtype=np.float32)
     g32 = r.uniform(0.5, 1.5, hidden).astype(np.float32)
     w32 = x32.copy()
-    samples.append(("rmsnorm_f32_64x4096", "full workload", 64, 2 * 64 * hidden * 4 + hidden * 4,
-                    lambda: L.isp_oracle_fused_norm_f32(None, w32.ctypes.data, None, g32.ctypes.data, 1e-5, 64,
-                                                        hidden, 0), lambda: w32.__setitem__(Ellipsis, x32)))
+    samples.append(dict(workload="rmsnorm_f32_64x4096", tokens=64, bytes=2 * 64 * hidden * 4 + hidden * 4,
+                        fn=lambda: L.isp_oracle_fused_norm_f32(None, p(w32), None, p(g32), 1e-5, 64, hidden, 0),
+                        reset=lambda: w32.__setitem__(Ellipsis, x32), sample="full workload",
+                        cache="1 MiB: cache-resident"))
+    # embedding: a random table, and different random ids on every repetition (the same ids again would
+    # turn the gather into a replay of 64 MiB of rows that a large L3 still holds)
     et, vocab = 8192, 32000
-    table = np.full((vocab, hidden), 0.01, f16)
-    ids = r.integers(0, vocab, et, dtype=np.int32)
+    table = r.integers(0, 0x3000, (vocab, hidden), dtype=np.uint16).view(f16)   # random finite bit patterns
+    id_sets = [r.integers(0, vocab, et, dtype=np.int32) for _ in range(8)]
     eo = np.empty((et, hidden), f16)
-    samples.append(("embedding_f16_8192x4096_v32000", "full workload", et, 2 * et * hidden * 2 + et * 4,
-                    lambda: L.isp_oracle_embedding(ids.ctypes.data, eo.ctypes.data, table.ctypes.data, et, hidden, 2),
-                    None))
-    qt, heads, hs, seq = 256, 96, 128, 512
+    turn = [0]
+
+    def gather():
+        ids = id_sets[turn[0] % len(id_sets)]
+        turn[0] += 1
+        L.isp_oracle_embedding(p(ids), p(eo), p(table), et, hidden, 2)
+    samples.append(dict(workload="embedding_f16_8192x4096_v32000", tokens=et, bytes=2 * et * hidden * 2 + et * 4,
+                        fn=gather, reset=None, sample="full workload, fresh random ids per repetition",
+                        cache="rows come from a 262 MB table (DRAM); the 64 MiB output is rewritten in place"))
+    # QKV + RoPE: the whole ragged batch
+    batch, seq, heads, hs = 8, 512, 96, 128
+    lens = np.ascontiguousarray(lens, dtype=np.int32)
+    qt = int(lens.sum())
     qkv, qb = normal(qt, heads, hs), normal(heads * hs, scale=0.02)
-    qo = [np.zeros((1, 32, seq, hs), f16) for _ in range(3)]
-    po, hist, ilen = np.zeros(qt, np.int32), np.zeros(1, np.int32), np.full(1, qt, np.int32)
-    samples.append(("qkv_bias_rope_transpose_f16_b8_s512", "one sequence of 256 tokens (of 2977)", qt,
-                    qt * (2 * heads * hs * 2 + 4) + heads * hs * 2,
-                    lambda: L.isp_oracle_qkv_rope_f16(qo[0].ctypes.data, qo[1].ctypes.data, qo[2].ctypes.data,
-                                                      qkv.ctypes.data, qb.ctypes.data, po.ctypes.data,
-                                                      hist.ctypes.data, ilen.ctypes.data, 1, seq, qt, 32, 32, hs,
-                                                      128, 10000.0), None))
-    st, inter = 256, 11008
-    sx, so = normal(st, 2, inter), np.empty((st, inter), f16)
-    samples.append(("swiglu_f16_decode_256x11008", "full workload (= 256 of the 8192 prefill tokens)", st,
-                    st * 3 * inter * 2,
-                    lambda: L.isp_oracle_swiglu_f16(sx.ctypes.data, so.ctypes.data, st, inter), None))
+    qo = [np.zeros((batch, 32, seq, hs), f16) for _ in range(3)]
+    po = np.repeat(np.concatenate([[0], np.cumsum(seq - lens)[:-1]]), lens).astype(np.int32)
+    hist = np.zeros(batch, np.int32)
+    samples.append(dict(workload="qkv_bias_rope_transpose_f16_b8_s512", tokens=qt,
+                        bytes=qt * (2 * heads * hs * 2 + 4) + heads * hs * 2 + 2 * batch * 4,
+                        fn=lambda: L.isp_oracle_qkv_rope_f16(p(qo[0]), p(qo[1]), p(qo[2]), p(qkv), p(qb), p(po), p(hist),
+                                                             p(lens), batch, seq, qt, 32, 32, hs, 128, 10000.0),
+                        reset=None, sample="full workload (8 sequences, %d tokens)" % qt,
+                        cache="compute-bound on the CPU (powf, cos, sin per element, as the reference's loop)"))
+    # SwiGLU prefill: all 8192 rows under OpenMP; one thread runs the first 1024 rows
+    inter, st_full, st_one = 11008, 8192, 1024
+    sx = np.empty((st_full, 2, inter), f16)
+    for i in range(0, st_full, 1024):
+        sx[i:i + 1024] = normal(1024, 2, inter)
+    so = np.empty((st_full, inter), f16)
+    samples.append(dict(workload="swiglu_f16_prefill_8192x11008", tokens=st_full, bytes=st_full * 3 * inter * 2,
+                        fn=lambda: L.isp_oracle_swiglu_f16(p(sx), p(so), st_full, inter), reset=None,
+                        one_fn=lambda: L.isp_oracle_swiglu_f16(p(sx), p(so), st_one, inter), one_tokens=st_one,
+                        one_bytes=st_one * 3 * inter * 2,
+                        sample="OpenMP: full workload; one thread: the first %d of %d rows" % (st_one, st_full),
+                        cache="541 MB: DRAM"))
+    sd = 256
+    samples.append(dict(workload="swiglu_f16_decode_256x11008", tokens=sd, bytes=sd * 3 * inter * 2,
+                        fn=lambda: L.isp_oracle_swiglu_f16(p(sx), p(so), sd, inter), reset=None,
+                        sample="full workload", cache="17 MB: cache-resident between repetitions"))
+    # padding offsets: the reference's serial loop (one thread by construction)
+    ppo, pcum = np.zeros((batch, seq), np.int32), np.zeros(batch + 1, np.int32)
+    samples.append(dict(workload="cal_padding_offset_b8_s512", tokens=qt, bytes=qt * 4 + (2 * batch + 1) * 4,
+                        fn=lambda: L.isp_oracle_cal_padding_offset(p(ppo), p(pcum), p(lens), batch, seq), reset=None,
+                        serial_only=True, sample="full workload", cache="12 KB: cache-resident"))
 
     def timed(fn, reset, threads, budget):
         o.set_threads(threads)
@@ -561,15 +608,20 @@ def cpu_baseline(budget_s):
         times.sort()
         return times[len(times) // 2], len(times)
 
-    cores = min(16, o.max_threads())
+    cores = o.max_threads()   # OMP_NUM_THREADS if set (the GPU box sets it to this job's CPU share), else all cores
     per = budget_s / (2.0 * len(samples))
     records = []
-    for name, what, toks, nbytes, fn, reset in samples:
-        t1, n1 = timed(fn, reset, 1, per * 1.4)
-        tn, nn = timed(fn, reset, cores, per * 0.6)
-        records.append({"workload": name, "sample": what, "kind": "port",
-                        "one_thread": {"GBps": nbytes / t1 / 1e9, "tokens_per_s": toks / t1, "cores": 1, "runs": n1},
-                        "openmp": {"GBps": nbytes / tn / 1e9, "tokens_per_s": toks / tn, "cores": cores, "runs": nn}})
+    for s in samples:
+        one_fn = s.get("one_fn", s["fn"])
+        t1, n1 = timed(one_fn, s["reset"], 1, per * 1.4)
+        b1, k1 = s.get("one_bytes", s["bytes"]), s.get("one_tokens", s["tokens"])
+        rec = {"workload": s["workload"], "sample": s["sample"], "kind": "port", "memory": s["cache"],
+               "one_thread": {"GBps": b1 / t1 / 1e9, "tokens_per_s": k1 / t1, "us": t1 * 1e6, "cores": 1, "runs": n1}}
+        if not s.get("serial_only"):
+            tn, nn = timed(s["fn"], s["reset"], cores, per * 0.6)
+            rec["openmp"] = {"GBps": s["bytes"] / tn / 1e9, "tokens_per_s": s["tokens"] / tn, "us": tn * 1e6,
+                             "cores": cores, "runs": nn}
+        records.append(rec)
     head = records[0]
     return {
         "value": head["one_thread"]["GBps"], "unit": "GB/s", "cores": 1, "kind": "port",
@@ -578,11 +630,25 @@ def cpu_baseline(budget_s):
         "tokens_per_s": head["one_thread"]["tokens_per_s"],
         "openmp": {"value": head["openmp"]["GBps"], "unit": "GB/s", "cores": cores,
                    "tokens_per_s": head["openmp"]["tokens_per_s"]},
+        "host_cpus": os.cpu_count(), "openmp_threads": cores,
         "per_kernel": records,
     }
 
 
 # --------------------------------------------------------------------------- main
+
+def compact(r):
+    """The per-workload record that travels inside `roofline.per_config`."""
+    out = {"kernel": r["kernel"], "us": round(r["ms_per_launch_events"] * 1e3, 3), "GBps": round(r["GBps"], 1),
+           "frac": round(r["frac_of_hbm_peak"], 4), "bytes": r["algorithmic_bytes"], "traffic": r["traffic"]}
+    if r.get("vs_copy") is not None:
+        out["vs_copy"] = round(r["vs_copy"], 3)
+    if r["tokens_per_s"]:
+        out["tokens_per_s"] = round(r["tokens_per_s"])
+    if r["launches_per_step"] != 1:
+        out["launches_per_step"] = r["launches_per_step"]
+    return out
+
 
 def main():
     a = parse()
@@ -600,6 +666,9 @@ def main():
     torch.manual_seed(0)
     stream = torch.cuda.Stream()
     handle = stream.cuda_stream
+    regions = region_count(a.steps, a.regions)
+    traffic = measured_traffic()
+    dispatch_log = []
 
     def run_all(rotate, names=None):
         out = []
@@ -611,7 +680,9 @@ def main():
             with torch.cuda.stream(stream):
                 w = make()
             torch.cuda.synchronize()
-            out.append(measure(torch, w, a.steps, a.warmup, stream))
+            r = measure(torch, w, a.steps, a.warmup, regions, stream, traffic)
+            out.append(r)
+            dispatch_log.append([name, w.kernel, r["launches_total"] * w.launches_per_step])
             # the buffers go back to torch's caching allocator, not to the driver: kernels that run
             # on freshly mapped device memory measured up to 2x slower at launch-bound sizes
             del w
@@ -626,6 +697,7 @@ def main():
             lib.isp_calibration_copy(b_buf.data_ptr(), a_buf.data_ptr(), 64 << 20, handle)
         stream.synchronize()
         del a_buf, b_buf
+    dispatch_log.append(["device_warmup", "isp::copy_vec<1>", 2000])
 
     if a.copy_curve:
         points = []
@@ -633,7 +705,7 @@ def main():
             with torch.cuda.stream(stream):
                 w = make_copy_workload(torch, lib, handle, (mib << 20) // 2)
             torch.cuda.synchronize()
-            r = measure(torch, w, a.steps, a.warmup, stream)
+            r = measure(torch, w, a.steps, a.warmup, regions, stream, traffic)
             points.append({"traffic_MiB": mib, "us_per_launch": r["ms_per_launch_events"] * 1e3, "GBps": r["GBps"],
                            "frac_of_hbm_peak": r["frac_of_hbm_peak"]})
             del w
@@ -659,48 +731,59 @@ def main():
         rate = (c_big["algorithmic_bytes"] - c_small["algorithmic_bytes"]) / (
             c_big["ms_per_launch_events"] - c_small["ms_per_launch_events"])          # bytes per ms
         fixed = c_small["ms_per_launch_events"] - c_small["algorithmic_bytes"] / rate  # ms
-        copy_model = {"fixed_us": fixed * 1e3, "asymptotic_GBps": rate / 1e6,
+        copy_model = {"fixed_us": round(fixed * 1e3, 3), "asymptotic_GBps": round(rate / 1e6, 1),
                       "form": "copy_time = fixed_us + bytes / asymptotic rate"}
         for r in results:
             t = fixed + r["algorithmic_bytes"] / rate
             r["copy_model_ms"] = t
             r["vs_copy"] = t / r["ms_per_launch_events"]
-    line = {
-        "metric": "HBM GB/s & % of peak per fused kernel at LLaMA-2-7B shapes; tokens/sec",
-        "value": head["GBps"], "unit": "GB/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
-        "ms_per_step": head["ms_per_step_wall"], "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-        "config": {"workload": head["workload"], "storage_dtype": "f16", "tokens_per_s": head["tokens_per_s"],
-                   "cache": "cold: launches rotate over %d buffer sets (> 1 GiB)" % head["buffer_sets"]},
-        "roofline": dict(head["roofline"], kernel=head["kernel"],
-                         algorithmic_bytes_per_launch=head["algorithmic_bytes"],
-                         avg_launch_ms=head["ms_per_launch_events"]),
-        "kernels": results,
-    }
+    config = {"workload": head["workload"], "storage_dtype": "f16", "tokens_per_s": head["tokens_per_s"],
+              "cache": "cold: launches rotate over %d buffer sets (> 1 GiB)" % head["buffer_sets"],
+              "timing": "median of %d back-to-back regions of %d launches, HIP events on the launch stream"
+                        % (regions, a.steps)}
     if copy_model:
-        line["copy_ceiling"] = copy_model
-    if not a.only:
+        config["copy_ceiling"] = copy_model
+    line = {}
+    if a.full:
+        line["kernels"] = results
+    if a.kernels_only:
+        line["dispatch_log"] = dispatch_log
+    if not a.only and not a.kernels_only:
         layer = context_layer_record(torch, a.steps, a.warmup, stream)
         own = {"qkv_bias_rope_transpose_f16_b8_s512": 1, "concat_kv_cache_f16_b8_q512_S1024": 1,
                "repeat_kv_cache_f16_b8_k512_S1024": 1, "transpose_remove_padding_f16_b8_s512": 1}
         tokens = layer["valid_tokens"]
         # fused norm (x2) and SwiGLU run on `tokens` rows here; scale their measured per-token cost
         est = sum(by_name[k]["ms_per_launch_events"] for k in own if k in by_name)
-        est += 2 * by_name["fused_add_bias_residual_rmsnorm_f16_2048x4096"]["ms_per_launch_events"] * tokens / 2048
+        est += 2 * by_name[HEADLINE]["ms_per_launch_events"] * tokens / 2048
         est += by_name["swiglu_f16_prefill_8192x11008"]["ms_per_launch_events"] * tokens / 8192
         layer["library_kernels_ms_estimate"] = est
         layer["library_kernels_share"] = est / layer["ms_per_layer"]
-        line["context_layer"] = layer
-        line["decode_sequence"] = decode_sequence_record(torch, stream)
-    # cache-resident rates (one buffer set, no rotation): the hot-path configurations by default, every
-    # workload with --warm.  These are not HBM rates: the 256 MB last-level cache serves part of them.
-    hot = None if a.warm else {
-        "fused_add_bias_residual_rmsnorm_f16_2048x4096", "rmsnorm_f32_64x4096", "embedding_f16_8192x4096_v32000",
-        "qkv_bias_rope_transpose_f16_b8_s512", "swiglu_f16_prefill_8192x11008", "swiglu_f16_decode_256x11008"}
-    line["warm_cache"] = {r["workload"]: {"GBps": r["GBps"], "ms_per_launch_events": r["ms_per_launch_events"]}
-                          for r in run_all(False, hot)}
-    if not a.no_cpu:
-        line["cpu_baseline"] = cpu_baseline(a.cpu_seconds)
+        config["context_layer"] = layer
+        config["decode_sequence"] = decode_sequence_record(torch, stream)
+    if not a.kernels_only:
+        # cache-resident rates (one buffer set, no rotation): the hot-path configurations by default, every
+        # workload with --warm.  These are not HBM rates: the 256 MB last-level cache serves part of them.
+        hot = None if a.warm else {
+            HEADLINE, "rmsnorm_f32_64x4096", "embedding_f16_8192x4096_v32000",
+            "qkv_bias_rope_transpose_f16_b8_s512", "swiglu_f16_prefill_8192x11008", "swiglu_f16_decode_256x11008"}
+        config["warm_cache_GBps"] = {r["workload"]: round(r["GBps"], 1) for r in run_all(False, hot)}
+    line.update({
+        "metric": "HBM GB/s & % of peak per fused kernel at LLaMA-2-7B shapes; tokens/sec",
+        "value": head["GBps"], "unit": "GB/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": head["ms_per_step_wall"], "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": config,
+        "roofline": {"bound": "hbm", "achieved": head["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": head["GBps"] / HBM_PEAK_GBS, "traffic": head["traffic"], "kernel": head["kernel"],
+                     "algorithmic_bytes_per_launch": head["algorithmic_bytes"],
+                     "avg_launch_ms": head["ms_per_launch_events"],
+                     "fastest_region_ms": head["ms_fastest_region"], "slowest_region_ms": head["ms_slowest_region"],
+                     "vs_copy": head.get("vs_copy"),
+                     "per_config": {r["workload"]: compact(r) for r in results}},
+    })
+    if not a.no_cpu and not a.kernels_only:
+        line["cpu_baseline"] = cpu_baseline(a.cpu_seconds, bench_lengths(torch).numpy())
     print(json.dumps(line))
 
 

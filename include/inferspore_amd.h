@@ -213,6 +213,14 @@ int isp_repeat_kv_cache_f16(const void* k_cache, const void* v_cache, void* k_ds
  *   results never depend on the knobs, only speed does.
  */
 int isp_calibration_copy(void* dst, const void* src, size_t bytes, isp_stream_t stream);
+/* isp_norm_launch_config: which instantiation isp_rmsnorm_* / isp_fused_add_bias_residual_rmsnorm_*
+ *   launch for `tokens` rows of `hidden` elements of `elem_size` bytes (2 or 4) on the vector path
+ *   (`fused` != 0: with a residual operand) -- waves per row, 16-byte vectors per lane, threads per
+ *   workgroup and store kind (0 plain, 1 non-temporal, 2 write-through), i.e. the template arguments
+ *   of isp::fused_norm_rows in a profiler trace.  Any output pointer may be NULL.  ISP_ERR_UNSUPPORTED
+ *   when the shape takes the scalar kernel. */
+int isp_norm_launch_config(int elem_size, int tokens, int hidden, int fused, int* waves_per_row,
+                           int* vectors_per_lane, int* block_threads, int* store_kind);
 
 typedef enum isp_tuning_knob {
     ISP_TUNE_NORM_WAVES_PER_ROW = 0, /* 1, 2, 4, 8 or 16 waves cooperate on one token row */
@@ -228,7 +236,9 @@ typedef enum isp_tuning_knob {
                                         workgroup; 0 = automatic: the fp16 one-vector-per-lane kernel where the shape
                                         allows it (128-element heads fully rotated, head counts multiples of 32),
                                         else the general kernel with 4 waves */
-    ISP_TUNE_COUNT = 8
+    ISP_TUNE_NORM_BLOCK_THREADS = 8, /* 256, 512 or 1024 threads per workgroup (several token rows share a
+                                        workgroup when a row needs fewer); 0 = automatic */
+    ISP_TUNE_COUNT = 9
 } isp_tuning_knob;
 int isp_tuning_set(int knob, int value);
 

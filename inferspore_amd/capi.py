@@ -13,7 +13,7 @@ ERR_LAUNCH = -4
 ERR_DEVICE = -5
 NORM_RESIDUAL_EXCLUDES_BIAS = 1
 (TUNE_NORM_WAVES_PER_ROW, TUNE_NORM_STORE, TUNE_SWIGLU_UNROLL, TUNE_SWIGLU_STORE, TUNE_EMBED_VARIANT,
- TUNE_EMBED_STORE, TUNE_QKV_STORE, TUNE_QKV_WAVES) = range(8)
+ TUNE_EMBED_STORE, TUNE_QKV_STORE, TUNE_QKV_WAVES, TUNE_NORM_BLOCK_THREADS) = range(9)
 
 _vp, _i, _f, _u = C.c_void_p, C.c_int, C.c_float, C.c_uint
 
@@ -44,6 +44,7 @@ SIGNATURES = {
     "isp_repeat_kv_cache_f16": (_i, [_vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i, _i, _i, _vp]),
     "isp_tuning_set": (_i, [_i, _i]),
     "isp_calibration_copy": (_i, [_vp, _vp, C.c_size_t, _vp]),
+    "isp_norm_launch_config": (_i, [_i, _i, _i, _i] + [C.POINTER(C.c_int)] * 4),
 }
 
 _lib = None

@@ -7,14 +7,16 @@
 // (the reference re-reads and read-modify-writes decoder_out); all global accesses are 16-byte
 // vectors; the row sum is a DPP wave reduction plus, when a row spans several waves, one small LDS
 // combine behind a single barrier, associated the same way under every launch configuration.
+#include <atomic>
+
 #include "isp_common.h"
 
 namespace isp {
 
-// One row is handled by WPR waves (ROW_THREADS = 64 * WPR lanes); a workgroup has at least 256
-// threads and therefore carries 4 / WPR rows when WPR < 4.  Each lane owns NV 16-byte vectors of
-// the row, strided by ROW_THREADS so that every load instruction of a wave covers 1 KiB of
-// contiguous memory.  ST is the store kind of the two outputs (non-temporal by default).
+// One row is handled by WPR waves (ROW_THREADS = 64 * WPR lanes); a workgroup of BLOCK threads
+// (256, 512 or 1024, at least one row) carries BLOCK / ROW_THREADS rows.  Each lane owns NV 16-byte
+// vectors of the row, strided by ROW_THREADS so that every load instruction of a wave covers 1 KiB
+// of contiguous memory.  ST is the store kind of the two outputs (non-temporal by default).
 constexpr int norm_block(int wpr) { return kWave * wpr > kBlock ? kWave * wpr : kBlock; }
 
 // p[0] + ... + p[N-1] as a balanced binary tree, neighbours first; N a power of two.
@@ -27,8 +29,8 @@ __device__ __forceinline__ float tree_sum(const float* p) {
     }
 }
 
-template <typename T, int NV, int WPR, int ST>
-__global__ __launch_bounds__(norm_block(WPR)) void fused_norm_rows(T* __restrict__ residual,
+template <typename T, int NV, int WPR, int ST, int BLOCK>
+__global__ __launch_bounds__(BLOCK) void fused_norm_rows(T* __restrict__ residual,
                                                                    T* __restrict__ out,
                                                                    const T* __restrict__ bias,
                                                                    const T* __restrict__ gamma,
@@ -36,7 +38,7 @@ __global__ __launch_bounds__(norm_block(WPR)) void fused_norm_rows(T* __restrict
                                                                    unsigned flags) {
     constexpr int VEC = Elem<T>::kVec;
     constexpr int ROW_THREADS = kWave * WPR;
-    constexpr int BLOCK = norm_block(WPR);
+    static_assert(BLOCK >= norm_block(WPR) && BLOCK % ROW_THREADS == 0, "workgroup must hold whole rows");
     constexpr int ROWS = BLOCK / ROW_THREADS;
 
     const int slot = threadIdx.x / ROW_THREADS;
@@ -177,41 +179,138 @@ __global__ __launch_bounds__(kBlock) void fused_norm_generic(T* residual, T* out
     }
 }
 
-template <typename T, int NV, int WPR, int ST>
-static hipError_t launch_rows(T* residual, T* out, const T* bias, const T* gamma, float eps,
-                              int tokens, int hidden, unsigned flags, hipStream_t s) {
-    constexpr int BLOCK = norm_block(WPR);
-    constexpr int ROWS = BLOCK / (kWave * WPR);
-    dim3 grid((unsigned)((tokens + ROWS - 1) / ROWS));
-    hipLaunchKernelGGL((fused_norm_rows<T, NV, WPR, ST>), grid, dim3(BLOCK), 0, s, residual, out,
-                       bias, gamma, eps, tokens, hidden, flags);
-    return hipGetLastError();
+// ----------------------------------------------------------------------------- launch
+constexpr int kMaxWpr = 16;  // 1024 threads
+constexpr int kMaxNv = 8;
+constexpr int kNvKinds = 4, kWprKinds = 5, kStoreKinds = 3, kBlockKinds = 2;
+
+template <typename T>
+using NormKernel = void (*)(T*, T*, const T*, const T*, float, int, int, unsigned);
+
+// One compiled instantiation: the kernel, its workgroup size and the rows a workgroup carries.
+template <typename T>
+struct NormVariant {
+    NormKernel<T> kernel;
+    int block, rows_per_block, index;
+};
+
+constexpr int log2_of(int v) { return v <= 1 ? 0 : 1 + log2_of(v / 2); }
+
+// BIG selects 512-thread workgroups for rows of up to four waves (two or more rows share a
+// workgroup); rows of 8 and 16 waves fill a workgroup on their own.
+template <typename T, int NV, int WPR, int ST, bool BIG>
+static NormVariant<T> variant_of() {
+    constexpr int MIN = norm_block(WPR);
+    constexpr int BLOCK = (BIG && MIN < 512) ? 512 : MIN;
+    constexpr int index = ((log2_of(NV) * kWprKinds + log2_of(WPR)) * kStoreKinds + ST) * kBlockKinds + (BIG ? 1 : 0);
+    return {fused_norm_rows<T, NV, WPR, ST, BLOCK>, BLOCK, BLOCK / (kWave * WPR), index};
 }
 
-template <typename T, int WPR, int ST>
-static hipError_t launch_rows_nv(int nv, T* residual, T* out, const T* bias, const T* gamma,
-                                 float eps, int tokens, int hidden, unsigned flags, hipStream_t s) {
-    if (nv <= 1) return launch_rows<T, 1, WPR, ST>(residual, out, bias, gamma, eps, tokens, hidden, flags, s);
-    if (nv <= 2) return launch_rows<T, 2, WPR, ST>(residual, out, bias, gamma, eps, tokens, hidden, flags, s);
-    if (nv <= 4) return launch_rows<T, 4, WPR, ST>(residual, out, bias, gamma, eps, tokens, hidden, flags, s);
-    return launch_rows<T, 8, WPR, ST>(residual, out, bias, gamma, eps, tokens, hidden, flags, s);
+template <typename T, int NV, int WPR>
+static NormVariant<T> variant_st(int st, bool big) {
+    if (st == kStoreThrough) return big ? variant_of<T, NV, WPR, kStoreThrough, true>() : variant_of<T, NV, WPR, kStoreThrough, false>();
+    if (st == kStoreStream) return big ? variant_of<T, NV, WPR, kStoreStream, true>() : variant_of<T, NV, WPR, kStoreStream, false>();
+    return big ? variant_of<T, NV, WPR, kStorePlain, true>() : variant_of<T, NV, WPR, kStorePlain, false>();
 }
 
-template <typename T, int ST>
-static hipError_t launch_rows_wpr(int wpr, int nv, T* residual, T* out, const T* bias,
-                                  const T* gamma, float eps, int tokens, int hidden, unsigned flags,
-                                  hipStream_t s) {
+template <typename T, int WPR>
+static NormVariant<T> variant_nv(int nv, int st, bool big) {
+    if (nv <= 1) return variant_st<T, 1, WPR>(st, big);
+    if (nv <= 2) return variant_st<T, 2, WPR>(st, big);
+    if (nv <= 4) return variant_st<T, 4, WPR>(st, big);
+    return variant_st<T, 8, WPR>(st, big);
+}
+
+// wpr in {1, 2, 4, 8, 16}; nv = vectors per lane (rounded up to 1, 2, 4 or 8 here).
+template <typename T>
+static NormVariant<T> norm_variant(int wpr, int nv, int st, bool big) {
     switch (wpr) {
-        case 1: return launch_rows_nv<T, 1, ST>(nv, residual, out, bias, gamma, eps, tokens, hidden, flags, s);
-        case 2: return launch_rows_nv<T, 2, ST>(nv, residual, out, bias, gamma, eps, tokens, hidden, flags, s);
-        case 4: return launch_rows_nv<T, 4, ST>(nv, residual, out, bias, gamma, eps, tokens, hidden, flags, s);
-        case 8: return launch_rows_nv<T, 8, ST>(nv, residual, out, bias, gamma, eps, tokens, hidden, flags, s);
-        default: return launch_rows_nv<T, 16, ST>(nv, residual, out, bias, gamma, eps, tokens, hidden, flags, s);
+        case 1: return variant_nv<T, 1>(nv, st, big);
+        case 2: return variant_nv<T, 2>(nv, st, big);
+        case 4: return variant_nv<T, 4>(nv, st, big);
+        case 8: return variant_nv<T, 8>(nv, st, big);
+        default: return variant_nv<T, 16>(nv, st, big);
     }
 }
 
-constexpr int kMaxWpr = 16;  // 1024 threads
-constexpr int kMaxNv = 8;
+// Token rows one launch of this instantiation keeps resident on the device at once: workgroups per
+// compute unit as the runtime's occupancy calculator reports them for the compiled kernel (its
+// register and LDS use decide), times compute units, times rows per workgroup.  Asked once per
+// instantiation and process; every device of one process is assumed to be the same gfx950 part.
+template <typename T>
+static long long resident_rows(const NormVariant<T>& v) {
+    static std::atomic<int> blocks_per_cu[kNvKinds * kWprKinds * kStoreKinds * kBlockKinds] = {};
+    int n = blocks_per_cu[v.index].load(std::memory_order_relaxed);
+    if (n == 0) {
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, reinterpret_cast<const void*>(v.kernel), v.block, 0) !=
+                hipSuccess || n <= 0) {
+            (void)hipGetLastError();
+            n = (kWave * 32) / v.block;  // 8 wavefronts per SIMD
+            if (n < 1) n = 1;
+        }
+        blocks_per_cu[v.index].store(n, std::memory_order_relaxed);
+    }
+    return (long long)n * (resident_waves() / 32) * v.rows_per_block;
+}
+
+struct NormPlan {
+    int wpr, nv, store, block_big;
+};
+
+// The launch configuration for `tokens` rows of `nvec` 16-byte vectors.
+template <typename T>
+static NormPlan plan_norm(int tokens, int nvec, bool fused) {
+    auto vectors_per_lane = [nvec](int w) { return (nvec + kWave * w - 1) / (kWave * w); };
+    // in place on both tensors: plain non-temporal stores measured best (write-through costs 2 %)
+    const int kind = store_kind(tuning(ISP_TUNE_NORM_STORE), kStoreStream);
+    const int block_knob = tuning(ISP_TUNE_NORM_BLOCK_THREADS);
+    int wpr = tuning(ISP_TUNE_NORM_WAVES_PER_ROW);
+    if (wpr != 1 && wpr != 2 && wpr != 4 && wpr != 8 && wpr != 16) {
+        // Automatic, from sweeps over 256..16384 rows of 4096 elements, both types:
+        //  * streaming regime (several rounds of waves): about two 16-byte loads in flight
+        //    per lane, i.e. waves per row = vectors x operand streams / 128, rounded to the
+        //    nearest power of two;
+        //  * if that needs more rows resident than the device holds at once, but fewer waves per
+        //    row fit the whole launch into a single round, take the single round: every load is
+        //    then issued at kernel start (5-10 % faster).  Whether a configuration fits is asked
+        //    of the occupancy calculator, because more vectors per lane mean more registers and
+        //    fewer resident waves (2 vectors per lane: 8 waves per SIMD, 4: 7, 8: 4);
+        //  * with a residual operand, a single round that is at least twice as large as it needs
+        //    to be to occupy half the machine: half the waves per row (two vectors of each
+        //    operand in flight per lane) measured 5 % faster;
+        //  * few rows: split rows further, down to one vector per lane, to occupy the machine.
+        const int streams = fused ? 2 : 1;
+        const int want = nvec * streams;  // 16-byte loads per row
+        wpr = 1;
+        while (wpr < kMaxWpr && 3 * kWave * wpr < want) wpr *= 2;  // 2^round(log2(want / 128))
+        while (wpr < kMaxWpr && vectors_per_lane(wpr) > kMaxNv) wpr *= 2;
+        auto fits = [&](int w) {
+            return vectors_per_lane(w) <= kMaxNv &&
+                   (long long)tokens <= resident_rows(norm_variant<T>(w, vectors_per_lane(w), kind, false));
+        };
+        if (!fits(wpr)) {
+            for (int w = wpr / 2; w >= 1 && vectors_per_lane(w) <= kMaxNv; w /= 2) {
+                if (fits(w)) {
+                    wpr = w;
+                    break;
+                }
+            }
+        } else {
+            const long long half = resident_waves() / 2;
+            while (wpr < kMaxWpr && vectors_per_lane(wpr) > 1 && (long long)tokens * wpr < half) wpr *= 2;
+            while (fused && wpr > 1 && (long long)tokens * (wpr / 2) >= half &&
+                   vectors_per_lane(wpr / 2) <= 2 && fits(wpr / 2))
+                wpr /= 2;
+        }
+    }
+    while (wpr < kMaxWpr && vectors_per_lane(wpr) > kMaxNv) wpr *= 2;
+    // 512-thread workgroups (two or four rows each) for 16-bit rows of two or four waves: half as
+    // many workgroups for the dispatcher to place before the last row's loads are out (+1 % at
+    // 2048 x 4096 with a residual, 0.5-3 % elsewhere; with 32-bit elements, and with one wave per
+    // row, the 256-thread workgroup measured 1-6 % faster)
+    const bool big = block_knob >= 512 || (block_knob <= 0 && (wpr == 4 || wpr == 2) && sizeof(T) == 2);
+    return {wpr, vectors_per_lane(wpr), kind, big ? 1 : 0};
+}
 
 template <typename T>
 static int fused_norm(void* residual_, void* out_, const void* bias_, const void* gamma_, float eps,
@@ -229,58 +328,45 @@ static int fused_norm(void* residual_, void* out_, const void* bias_, const void
     const bool vec_ok = (hidden % VEC == 0) && aligned16(out) && aligned16(gamma) &&
                         (!residual || aligned16(residual)) && (!bias || aligned16(bias)) &&
                         (hidden / VEC) <= kMaxNv * kWave * kMaxWpr;
-    hipError_t e;
     if (!vec_ok) {
         hipLaunchKernelGGL((fused_norm_generic<T>), dim3((unsigned)tokens), dim3(kBlock), 0, s,
                            residual, out, bias, gamma, eps, tokens, hidden, flags);
-        e = hipGetLastError();
     } else {
-        const int nvec = hidden / VEC;
-        auto vectors_per_lane = [nvec](int w) { return (nvec + kWave * w - 1) / (kWave * w); };
-        int wpr = tuning(ISP_TUNE_NORM_WAVES_PER_ROW);
-        if (wpr != 1 && wpr != 2 && wpr != 4 && wpr != 8 && wpr != 16) {
-            // Automatic, from sweeps over 512..16384 rows of 2048..8192 elements, both types:
-            //  * streaming regime (several rounds of waves): about two 16-byte loads in flight
-            //    per lane, i.e. waves per row = vectors x operand streams / 128, rounded to the
-            //    nearest power of two;
-            //  * if that needs more waves than the device holds at once, but fewer waves per row
-            //    (at most 4 vectors per lane) fit the whole launch into a single round, take the
-            //    single round: every load is then issued at kernel start (5-10 % faster);
-            //  * few rows: split rows further, down to one vector per lane, to occupy the machine.
-            const int streams = residual ? 2 : 1;
-            const int want = nvec * streams;  // 16-byte loads per row
-            wpr = 1;
-            while (wpr < kMaxWpr && 3 * kWave * wpr < want) wpr *= 2;  // 2^round(log2(want / 128))
-            const long long capacity = resident_waves();
-            if ((long long)tokens * wpr > capacity) {
-                for (int w = wpr / 2; w >= 1; w /= 2) {
-                    if ((long long)tokens * w <= capacity) {
-                        if (vectors_per_lane(w) <= 4) wpr = w;
-                        break;
-                    }
-                }
-            } else {
-                while (wpr < kMaxWpr && vectors_per_lane(wpr) > 1 && (long long)tokens * wpr < capacity / 2)
-                    wpr *= 2;
-            }
-        }
-        while (wpr < kMaxWpr && vectors_per_lane(wpr) > kMaxNv) wpr *= 2;
-        const int nv = vectors_per_lane(wpr);
-        // in place on both tensors: plain non-temporal stores measured best (write-through costs 2 %)
-        const int kind = store_kind(tuning(ISP_TUNE_NORM_STORE), kStoreStream);
-        if (kind == kStoreThrough)
-            e = launch_rows_wpr<T, kStoreThrough>(wpr, nv, residual, out, bias, gamma, eps, tokens, hidden, flags, s);
-        else if (kind == kStoreStream)
-            e = launch_rows_wpr<T, kStoreStream>(wpr, nv, residual, out, bias, gamma, eps, tokens, hidden, flags, s);
-        else
-            e = launch_rows_wpr<T, kStorePlain>(wpr, nv, residual, out, bias, gamma, eps, tokens, hidden, flags, s);
+        const NormPlan plan = plan_norm<T>(tokens, hidden / VEC, residual != nullptr);
+        const NormVariant<T> v = norm_variant<T>(plan.wpr, plan.nv, plan.store, plan.block_big != 0);
+        const dim3 grid((unsigned)((tokens + v.rows_per_block - 1) / v.rows_per_block));
+        hipLaunchKernelGGL(v.kernel, grid, dim3(v.block), 0, s, residual, out, bias, gamma, eps,
+                           tokens, hidden, flags);
     }
-    return note_launch(e);
+    return note_launch(hipGetLastError());
+}
+
+template <typename T>
+static int describe_plan(int tokens, int hidden, int fused, int* wpr, int* nv, int* block, int* store) {
+    constexpr int VEC = Elem<T>::kVec;
+    if (tokens <= 0 || hidden <= 0) return ISP_ERR_BAD_SHAPE;
+    if (hidden % VEC != 0 || hidden / VEC > kMaxNv * kWave * kMaxWpr) return ISP_ERR_UNSUPPORTED;
+    const NormPlan plan = plan_norm<T>(tokens, hidden / VEC, fused != 0);
+    const NormVariant<T> v = norm_variant<T>(plan.wpr, plan.nv, plan.store, plan.block_big != 0);
+    if (wpr) *wpr = plan.wpr;
+    if (nv) *nv = plan.nv <= 1 ? 1 : plan.nv <= 2 ? 2 : plan.nv <= 4 ? 4 : 8;
+    if (block) *block = v.block;
+    if (store) *store = plan.store;
+    return ISP_OK;
 }
 
 }  // namespace isp
 
 extern "C" {
+
+int isp_norm_launch_config(int elem_size, int tokens, int hidden, int fused, int* waves_per_row,
+                           int* vectors_per_lane, int* block_threads, int* store_kind) {
+    if (elem_size == 2)
+        return isp::describe_plan<__half>(tokens, hidden, fused, waves_per_row, vectors_per_lane, block_threads, store_kind);
+    if (elem_size == 4)
+        return isp::describe_plan<float>(tokens, hidden, fused, waves_per_row, vectors_per_lane, block_threads, store_kind);
+    return ISP_ERR_BAD_SHAPE;
+}
 
 int isp_fused_add_bias_residual_rmsnorm_f32(void* residual, void* decoder_out, const void* bias,
                                             const void* gamma, float eps, int tokens, int hidden,

@@ -38,12 +38,12 @@ def with_knobs(settings, fn):
 
 
 @pytest.mark.parametrize("dtype", [np.float16, np.float32])
-def test_norm_every_vectors_per_lane_waves_per_row_and_store_kind(isp, oracle, dtype):
+def test_norm_every_vectors_per_lane_waves_per_row_store_kind_and_workgroup_size(isp, oracle, dtype):
     from inferspore_amd import capi
     vec = 8 if dtype == np.float16 else 4
     for wpr, nv in itertools.product((1, 2, 4, 8, 16), (1, 2, 4, 8)):
         hidden = vec * 64 * wpr * nv - (vec if nv > 1 else 0)  # just inside nv vectors per lane, ragged last vector
-        tokens = 5
+        tokens = 7  # not a multiple of the 2, 4 or 8 rows a workgroup carries
         res, out, bias, gamma = norm_inputs(tokens, hidden, dtype, seed=wpr * 10 + nv)
         d_bias, d_gamma = dev(bias), dev(gamma)
 
@@ -60,9 +60,10 @@ def test_norm_every_vectors_per_lane_waves_per_row_and_store_kind(isp, oracle, d
         else:
             assert_f16_close(base[1], e_out, "norm hidden %d" % hidden, max_mismatch_fraction=0.05)
         # the row sum is one fixed tree whatever the split of the row over waves and vectors per lane
-        for split, store in itertools.product((1, 2, 4, 8, 16), (1, 2, 3)):
-            say("norm %s hidden=%d waves/row=%d store=%d" % (dtype.__name__, hidden, split, store))
-            got = with_knobs({capi.TUNE_NORM_WAVES_PER_ROW: split, capi.TUNE_NORM_STORE: store}, run)
+        for split, store, block in itertools.product((1, 2, 4, 8, 16), (1, 2, 3), (256, 512)):
+            say("norm %s hidden=%d waves/row=%d store=%d block=%d" % (dtype.__name__, hidden, split, store, block))
+            got = with_knobs({capi.TUNE_NORM_WAVES_PER_ROW: split, capi.TUNE_NORM_STORE: store,
+                              capi.TUNE_NORM_BLOCK_THREADS: block}, run)
             assert np.array_equal(got[0], base[0]) and np.array_equal(got[1], base[1])
 
 
