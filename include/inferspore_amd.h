@@ -238,7 +238,9 @@ typedef enum isp_tuning_knob {
                                         else the general kernel with 4 waves */
     ISP_TUNE_NORM_BLOCK_THREADS = 8, /* 256, 512 or 1024 threads per workgroup (several token rows share a
                                         workgroup when a row needs fewer); 0 = automatic */
-    ISP_TUNE_COUNT = 9
+    ISP_TUNE_NORM_ORDER = 9,         /* 2 = streaming (each vector processed, and the residual stored, as it
+                                        arrives); 0, 1 = read everything, then write everything (default) */
+    ISP_TUNE_COUNT = 10
 } isp_tuning_knob;
 int isp_tuning_set(int knob, int value);
 

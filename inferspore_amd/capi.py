@@ -13,7 +13,7 @@ ERR_LAUNCH = -4
 ERR_DEVICE = -5
 NORM_RESIDUAL_EXCLUDES_BIAS = 1
 (TUNE_NORM_WAVES_PER_ROW, TUNE_NORM_STORE, TUNE_SWIGLU_UNROLL, TUNE_SWIGLU_STORE, TUNE_EMBED_VARIANT,
- TUNE_EMBED_STORE, TUNE_QKV_STORE, TUNE_QKV_WAVES, TUNE_NORM_BLOCK_THREADS) = range(9)
+ TUNE_EMBED_STORE, TUNE_QKV_STORE, TUNE_QKV_WAVES, TUNE_NORM_BLOCK_THREADS, TUNE_NORM_ORDER) = range(10)
 
 _vp, _i, _f, _u = C.c_void_p, C.c_int, C.c_float, C.c_uint
 

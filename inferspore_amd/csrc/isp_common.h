@@ -122,6 +122,21 @@ struct Elem<float> {
     }
     __device__ static __forceinline__ float to_f32(float x) { return x; }
     __device__ static __forceinline__ float from_f32(float x) { return x; }
+    __device__ static __forceinline__ float pinned(float x) { return x; }
+    __device__ static __forceinline__ vec16 pack_pinned(const float* f) { return pack(f); }
+    // x = a + b,  x += b,  y = g * x  on one vector, element by element in fp32
+    __device__ static __forceinline__ void sum(const vec16& a, const vec16& b, float* x) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) x[i] = __uint_as_float(a.w[i]) + __uint_as_float(b.w[i]);
+    }
+    __device__ static __forceinline__ void accumulate(const vec16& b, float* x) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) x[i] += __uint_as_float(b.w[i]);
+    }
+    __device__ static __forceinline__ void scale(const vec16& g, const float* x, float* y) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) y[i] = __uint_as_float(g.w[i]) * x[i];
+    }
 };
 
 template <>
@@ -153,8 +168,58 @@ struct Elem<__half> {
         }
         return v;
     }
+    // For values that went through pinned() when they were produced and are used again afterwards:
+    // pinning them a second time here would cost a register copy each.
+    __device__ static __forceinline__ vec16 pack_pinned(const float* f) {
+        vec16 v;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            __half2 h = __floats2half2_rn(f[2 * i], f[2 * i + 1]);
+            v.w[i] = *reinterpret_cast<const uint32_t*>(&h);
+        }
+        return v;
+    }
     __device__ static __forceinline__ float to_f32(__half x) { return __half2float(x); }
     __device__ static __forceinline__ __half from_f32(float x) { return __float2half_rn(pinned(x)); }
+    // x = a + b,  x += b,  y = g * x  on one vector, element by element in fp32.  Written as
+    // fma(half, 1, .) / fma(half, x, -0) with the constants hidden from the optimiser: the compiler
+    // then emits one mixed-precision multiply-add that reads the fp16 operand directly, in place of
+    // a conversion plus an add or multiply -- same value (the product with 1 and the sum with -0 are
+    // exact), a third of the instructions.
+    __device__ static __forceinline__ float lo(uint32_t w) {
+        return __half2float(__ushort_as_half((unsigned short)(w & 0xffffu)));
+    }
+    __device__ static __forceinline__ float hi(uint32_t w) {
+        return __half2float(__ushort_as_half((unsigned short)(w >> 16)));
+    }
+    __device__ static __forceinline__ float hidden_constant(float v) {
+        asm volatile("" : "+v"(v));
+        return v;
+    }
+    __device__ static __forceinline__ void sum(const vec16& a, const vec16& b, float* x) {
+        const float one = hidden_constant(1.0f);
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            x[2 * i] = __fmaf_rn(lo(a.w[i]), one, lo(b.w[i]));
+            x[2 * i + 1] = __fmaf_rn(hi(a.w[i]), one, hi(b.w[i]));
+        }
+    }
+    __device__ static __forceinline__ void accumulate(const vec16& b, float* x) {
+        const float one = hidden_constant(1.0f);
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            x[2 * i] = __fmaf_rn(lo(b.w[i]), one, x[2 * i]);
+            x[2 * i + 1] = __fmaf_rn(hi(b.w[i]), one, x[2 * i + 1]);
+        }
+    }
+    __device__ static __forceinline__ void scale(const vec16& g, const float* x, float* y) {
+        const float negzero = hidden_constant(-0.0f);
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            y[2 * i] = __fmaf_rn(lo(g.w[i]), x[2 * i], negzero);
+            y[2 * i + 1] = __fmaf_rn(hi(g.w[i]), x[2 * i + 1], negzero);
+        }
+    }
 };
 
 // DPP lane exchange inside the VALU (no LDS traffic).  `ctrl` is the DPP control word.

@@ -29,13 +29,30 @@ __device__ __forceinline__ float tree_sum(const float* p) {
     }
 }
 
+// The order of the memory operations is the design, and each step of it is measured (2048 x 4096 fp16
+// with residual and bias, 67 MB per launch, one round of waves; alternating builds on one device):
+//   1. all streamed vectors of the lane are requested at kernel entry;
+//   2. nothing is computed or requested until ALL of them have arrived (starting on the first vector
+//      while the others are in flight: 12.9 us instead of 11.0 us);
+//   3. bias is requested only then, one vector at a time, where it is consumed, and gamma after the
+//      row has been summed (either of them requested together with the rows, or both bias vectors
+//      at once: 12.6-12.8 us -- every workgroup then hits the same few L2 lines at the same time);
+//   4. every store is issued at the very end, behind the barrier, after gamma has arrived (the
+//      residual stored inside the loop, as soon as it is known: 11.7 us; a store followed by a
+//      wait for a later load also makes the wave wait for the store's acknowledgement, because
+//      loads and stores share one in-order counter).
+// The common factor of 2-4: the device reaches its best rate when the launch first reads and then
+// writes; writes that start while most reads are still queued cost more than the idle registers.
+// The opposite order -- start on each vector as it arrives, store the residual as soon as it is known
+// -- stays selectable (kNormStreamingOrder, an internal flag bit the launcher sets from a tuning
+// knob): with several rounds of waves it measured within 1 % of the order above for 16-bit rows and
+// plain RMSNorm, and 8-12 % slower for 32-bit rows with a residual.  Same bits under both.
+constexpr unsigned kNormStreamingOrder = 0x80000000u;
+
 template <typename T, int NV, int WPR, int ST, int BLOCK>
-__global__ __launch_bounds__(BLOCK) void fused_norm_rows(T* __restrict__ residual,
-                                                                   T* __restrict__ out,
-                                                                   const T* __restrict__ bias,
-                                                                   const T* __restrict__ gamma,
-                                                                   float eps, int tokens, int hidden,
-                                                                   unsigned flags) {
+__global__ __launch_bounds__(BLOCK) void fused_norm_rows(T* residual, T* out, const T* bias,
+                                                         const T* gamma, float eps, int tokens,
+                                                         int hidden, unsigned flags) {
     constexpr int VEC = Elem<T>::kVec;
     constexpr int ROW_THREADS = kWave * WPR;
     static_assert(BLOCK >= norm_block(WPR) && BLOCK % ROW_THREADS == 0, "workgroup must hold whole rows");
@@ -46,9 +63,12 @@ __global__ __launch_bounds__(BLOCK) void fused_norm_rows(T* __restrict__ residua
     const int row = blockIdx.x * ROWS + slot;
     const bool live = row < tokens;  // uniform within a wave
     const int nvec = hidden / VEC;
+    const bool has_res = residual != nullptr, has_bias = bias != nullptr;  // uniform: scalar branches
+    const bool literal_order = (flags & ISP_NORM_RESIDUAL_EXCLUDES_BIAS) != 0;
+    const bool streaming = (flags & kNormStreamingOrder) != 0;
     const size_t base = (size_t)(live ? row : 0) * (size_t)hidden;
     T* out_row = out + base;
-    T* rsd_row = residual ? residual + base : nullptr;
+    T* rsd_row = residual + base;  // dereferenced only when has_res
 
     vec16 vo[NV], vr[NV];
     bool ok[NV];
@@ -58,14 +78,16 @@ __global__ __launch_bounds__(BLOCK) void fused_norm_rows(T* __restrict__ residua
         ok[j] = live && vi < nvec;
         if (ok[j]) {
             vo[j] = load16_stream(out_row + (size_t)vi * VEC);
-            if (rsd_row) vr[j] = load16_stream(rsd_row + (size_t)vi * VEC);
+            if (has_res) vr[j] = load16_stream(rsd_row + (size_t)vi * VEC);
         }
     }
+    // step 2: the empty asm uses the loaded registers (so the wait for them is placed here) and
+    // nothing that touches memory may be moved across it
+    if (!streaming) {
+#pragma unroll
+        for (int j = 0; j < NV; j++) asm volatile("" : "+v"(vo[j].w[0]), "+v"(vr[j].w[0]) : : "memory");
+    }
 
-    // bias and gamma are deliberately not requested up front with the rows: issued at kernel start,
-    // every workgroup hits the same few L2 lines at once and the streaming loads queue up behind them
-    // (measured: 13.3 us instead of 11.7 us at 2048 x 4096 fp16).  bias is loaded where it is used,
-    // gamma once the row has been summed (below).
     float x[NV][VEC];
     float part[NV];  // sum of squares of each of this lane's vectors
 #pragma unroll
@@ -73,34 +95,37 @@ __global__ __launch_bounds__(BLOCK) void fused_norm_rows(T* __restrict__ residua
         part[j] = 0.0f;
         if (ok[j]) {
             const int vi = lane + j * ROW_THREADS;
-            Elem<T>::unpack(vo[j], x[j]);
-            if (rsd_row) {
-                float r[VEC];
-                Elem<T>::unpack(vr[j], r);
-#pragma unroll
-                for (int e = 0; e < VEC; e++) x[j][e] += r[e];
-                if (flags & ISP_NORM_RESIDUAL_EXCLUDES_BIAS)
-                    store16_sel<ST>(rsd_row + (size_t)vi * VEC, Elem<T>::pack(x[j]));
-            }
-            if (bias) {
-                float b[VEC];
-                Elem<T>::unpack(load16(bias + (size_t)vi * VEC), b);
-#pragma unroll
-                for (int e = 0; e < VEC; e++) x[j][e] += b[e];
-            }
-            if (rsd_row && !(flags & ISP_NORM_RESIDUAL_EXCLUDES_BIAS))
+            vec16 vb;
+            if (has_bias) vb = load16(bias + (size_t)vi * VEC);
+            asm volatile("" ::: "memory");  // step 3: the next vector's bias is not requested early
+            if (has_res) Elem<T>::sum(vo[j], vr[j], x[j]);
+            else Elem<T>::unpack(vo[j], x[j]);
+            if (has_res && literal_order) {
+                // the reference's literal order stores the residual before the bias is added; that
+                // mode keeps its store here (x does not survive the addition of the bias)
                 store16_sel<ST>(rsd_row + (size_t)vi * VEC, Elem<T>::pack(x[j]));
+            }
+            if (has_bias) Elem<T>::accumulate(vb, x[j]);
+            // x is stored (rounded to T) and also used further in fp32: the value is fixed in its
+            // register here so that the rounding of the store cannot be merged with this sum
 #pragma unroll
-            for (int e = 0; e < VEC; e++) part[j] += x[j][e] * x[j][e];
+            for (int e = 0; e < VEC; e++) x[j][e] = Elem<T>::pinned(x[j][e]);
+            if (has_res && streaming && !literal_order)
+                store16_sel<ST>(rsd_row + (size_t)vi * VEC, Elem<T>::pack_pinned(x[j]));
+            // one product and then fused multiply-adds in element order: no freedom for the compiler
+            // in how it contracts the sum, so every instantiation associates it the same way
+            float p = x[j][0] * x[j][0];
+#pragma unroll
+            for (int e = 1; e < VEC; e++) p = __fmaf_rn(x[j][e], x[j][e], p);
+            part[j] = p;
         }
-        // With two vectors per lane the first is reduced over the wave here, not after the loop: the
-        // vectors arrive in order, and its reduction then runs while the second is still on its
-        // way (with four or more, waiting for them one by one costs more than it hides).
+        // with one or two vectors per lane each is reduced over the wave as soon as it is summed,
+        // underneath the round trip of the next bias vector
         if (NV <= 2) part[j] = wave_sum(part[j]);
     }
 
-    // gamma is requested once this lane's part of the row has arrived and been summed: the L2 round
-    // trip then overlaps the reduction and the barrier instead of following them
+    // gamma is requested once this lane's part of the row has been summed: the L2 round trip then
+    // overlaps the reduction and the barrier instead of following them
     vec16 vg[NV];
 #pragma unroll
     for (int j = 0; j < NV; j++) {
@@ -130,16 +155,24 @@ __global__ __launch_bounds__(BLOCK) void fused_norm_rows(T* __restrict__ residua
     const float total = tree_sum<NV>(part);
     const float inv = rsqrtf(total / (float)hidden + eps);
 
+    // step 4: gamma has arrived before the first store is issued, so no wait below falls behind a store
+#pragma unroll
+    for (int j = 0; j < NV; j++) asm volatile("" : "+v"(vg[j].w[0]) : : "memory");
+    if (has_res && !literal_order && !streaming) {
+#pragma unroll
+        for (int j = 0; j < NV; j++) {
+            if (ok[j])
+                store16_sel<ST>(rsd_row + (size_t)(lane + j * ROW_THREADS) * VEC, Elem<T>::pack_pinned(x[j]));
+        }
+    }
 #pragma unroll
     for (int j = 0; j < NV; j++) {
         if (ok[j]) {
-            const int vi = lane + j * ROW_THREADS;
-            float g[VEC];
-            Elem<T>::unpack(vg[j], g);
             float y[VEC];
+            Elem<T>::scale(vg[j], x[j], y);
 #pragma unroll
-            for (int e = 0; e < VEC; e++) y[e] = g[e] * x[j][e] * inv;
-            store16_sel<ST>(out_row + (size_t)vi * VEC, Elem<T>::pack(y));
+            for (int e = 0; e < VEC; e++) y[e] *= inv;
+            store16_sel<ST>(out_row + (size_t)(lane + j * ROW_THREADS) * VEC, Elem<T>::pack(y));
         }
     }
 }
@@ -255,6 +288,7 @@ static long long resident_rows(const NormVariant<T>& v) {
 
 struct NormPlan {
     int wpr, nv, store, block_big;
+    bool streaming;  // kNormStreamingOrder
 };
 
 // The launch configuration for `tokens` rows of `nvec` 16-byte vectors.
@@ -309,7 +343,8 @@ static NormPlan plan_norm(int tokens, int nvec, bool fused) {
     // 2048 x 4096 with a residual, 0.5-3 % elsewhere; with 32-bit elements, and with one wave per
     // row, the 256-thread workgroup measured 1-6 % faster)
     const bool big = block_knob >= 512 || (block_knob <= 0 && (wpr == 4 || wpr == 2) && sizeof(T) == 2);
-    return {wpr, vectors_per_lane(wpr), kind, big ? 1 : 0};
+    const bool streaming = tuning(ISP_TUNE_NORM_ORDER) == 2;
+    return {wpr, vectors_per_lane(wpr), kind, big ? 1 : 0, streaming};
 }
 
 template <typename T>
@@ -330,13 +365,14 @@ static int fused_norm(void* residual_, void* out_, const void* bias_, const void
                         (hidden / VEC) <= kMaxNv * kWave * kMaxWpr;
     if (!vec_ok) {
         hipLaunchKernelGGL((fused_norm_generic<T>), dim3((unsigned)tokens), dim3(kBlock), 0, s,
-                           residual, out, bias, gamma, eps, tokens, hidden, flags);
+                           residual, out, bias, gamma, eps, tokens, hidden, flags & ~kNormStreamingOrder);
     } else {
         const NormPlan plan = plan_norm<T>(tokens, hidden / VEC, residual != nullptr);
         const NormVariant<T> v = norm_variant<T>(plan.wpr, plan.nv, plan.store, plan.block_big != 0);
         const dim3 grid((unsigned)((tokens + v.rows_per_block - 1) / v.rows_per_block));
         hipLaunchKernelGGL(v.kernel, grid, dim3(v.block), 0, s, residual, out, bias, gamma, eps,
-                           tokens, hidden, flags);
+                           tokens, hidden,
+                           (flags & ~kNormStreamingOrder) | (plan.streaming ? kNormStreamingOrder : 0u));
     }
     return note_launch(hipGetLastError());
 }

@@ -60,10 +60,11 @@ def test_norm_every_vectors_per_lane_waves_per_row_store_kind_and_workgroup_size
         else:
             assert_f16_close(base[1], e_out, "norm hidden %d" % hidden, max_mismatch_fraction=0.05)
         # the row sum is one fixed tree whatever the split of the row over waves and vectors per lane
-        for split, store, block in itertools.product((1, 2, 4, 8, 16), (1, 2, 3), (256, 512)):
-            say("norm %s hidden=%d waves/row=%d store=%d block=%d" % (dtype.__name__, hidden, split, store, block))
+        for split, store, block, order in itertools.product((1, 2, 4, 8, 16), (1, 2, 3), (256, 512), (1, 2)):
+            say("norm %s hidden=%d waves/row=%d store=%d block=%d order=%d" % (dtype.__name__, hidden, split, store,
+                                                                                 block, order))
             got = with_knobs({capi.TUNE_NORM_WAVES_PER_ROW: split, capi.TUNE_NORM_STORE: store,
-                              capi.TUNE_NORM_BLOCK_THREADS: block}, run)
+                              capi.TUNE_NORM_BLOCK_THREADS: block, capi.TUNE_NORM_ORDER: order}, run)
             assert np.array_equal(got[0], base[0]) and np.array_equal(got[1], base[1])
 
 
