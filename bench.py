@@ -218,7 +218,7 @@ def make_workloads(torch, lib, stream_handle, rotate):
         batch, seq, tokens, lens_d, po = padded_batch()
         w.name, w.dtype, w.tokens = "qkv_bias_rope_transpose_%s_b8_s512%s" % (sfx, tag), sfx, tokens
         if es == 2 and hs == 128 and hn % 32 == 0 and kvn % 32 == 0:
-            w.kernel = "isp::qkv_rope_lean_f16<2, true>"
+            w.kernel = "isp::qkv_rope_lean_f16<2, true, false>"
         else:
             w.kernel = "isp::qkv_rope_wave<%s, %d, 2, 4>" % ("__half" if es == 2 else "float", hs)
         w.bytes_per_launch = tokens * (2 * (hn + 2 * kvn) * hs * es + 4) + (hn + 2 * kvn) * hs * es + 2 * batch * 4
@@ -237,6 +237,47 @@ def make_workloads(torch, lib, stream_handle, rotate):
         w.reset = lambda: None
         w.config = {"batch": batch, "max_seq": seq, "valid_tokens": tokens, "heads": "%dq/%dkv" % (hn, kvn),
                     "head_dim": hs}
+        return w
+
+    def qkv_append(fused):
+        """QKV step + KV-cache append at the benchmark shape: one fused launch (k and v rows written to the
+        cache only), or the two launches it replaces.  Both are priced at the bytes the fused form has
+        to move (packed qkv read once; q and the cache rows written once)."""
+        w = Workload()
+        tdtype, es, hn, kvn, hs, max_seq = torch.float16, 2, 32, 32, 128, 1024
+        batch, seq, tokens, lens_d, po = padded_batch()
+        w.dtype, w.tokens = "f16", tokens
+        w.bytes_per_launch = tokens * (2 * (hn + 2 * kvn) * hs * es + 4) + (hn + 2 * kvn) * hs * es + 3 * batch * 4
+        hist = torch.zeros(batch, device=dev, dtype=torch.int32)
+        bias = (0.02 * torch.randn((hn + 2 * kvn) * hs, device=dev)).to(tdtype)
+        set_bytes = tokens * (hn + 2 * kvn) * hs * es + batch * hn * seq * hs * es + 2 * batch * kvn * max_seq * hs * es
+        if not fused:
+            set_bytes += 2 * batch * kvn * seq * hs * es
+        R = w.sets_for(set_bytes, rotate)
+        ins = [torch.randn((tokens, hn + 2 * kvn, hs), device=dev).to(tdtype) for _ in range(R)]
+        qs = [torch.zeros((batch, hn, seq, hs), device=dev, dtype=tdtype) for _ in range(R)]
+        caches = [[torch.zeros((1, batch, kvn, max_seq, hs), device=dev, dtype=tdtype) for _ in range(2)] for _ in range(R)]
+        w.keep = (lens_d, po, hist, bias, ins, qs, caches)
+        if fused:
+            w.name, w.kernel = "qkv_bias_rope_transpose_append_f16_b8_s512_S1024", "isp::qkv_rope_lean_f16<2, true, true>"
+            w.bind(lib.isp_qkv_bias_rope_transpose_append_f16,
+                   [(qs[j].data_ptr(), None, None, caches[j][0].data_ptr(), caches[j][1].data_ptr(), 0, max_seq,
+                     ins[j].data_ptr(), bias.data_ptr(), po.data_ptr(), hist.data_ptr(), lens_d.data_ptr(), batch, seq,
+                     tokens, hn, kvn, hs, hs, 10000.0, st) for j in range(R)])
+        else:
+            w.name = "qkv_bias_rope_transpose_then_concat_kv_f16_b8_s512_S1024"
+            w.kernel = "isp::qkv_rope_lean_f16<2, true, false> + isp::concat_kv_vec<256>"
+            kvs = [[torch.zeros((batch, kvn, seq, hs), device=dev, dtype=tdtype) for _ in range(2)] for _ in range(R)]
+            w.keep += (kvs,)
+            w.bind_pair(lib.isp_qkv_bias_rope_transpose_f16,
+                        [(qs[j].data_ptr(), kvs[j][0].data_ptr(), kvs[j][1].data_ptr(), ins[j].data_ptr(),
+                          bias.data_ptr(), po.data_ptr(), hist.data_ptr(), lens_d.data_ptr(), batch, seq, tokens, hn,
+                          kvn, hs, hs, 10000.0, 2048, 0, st) for j in range(R)],
+                        lib.isp_concat_kv_cache_f16,
+                        [(kvs[j][0].data_ptr(), kvs[j][1].data_ptr(), caches[j][0].data_ptr(), caches[j][1].data_ptr(),
+                          0, lens_d.data_ptr(), hist.data_ptr(), batch, kvn, seq, max_seq, hs, st) for j in range(R)])
+        w.reset = lambda: None
+        w.config = {"batch": batch, "max_seq": seq, "valid_tokens": tokens, "max_seq_len": max_seq}
         return w
 
     def swiglu(tokens, tag, tdtype=torch.float16):
@@ -289,13 +330,13 @@ def make_workloads(torch, lib, stream_handle, rotate):
                   for _ in range(R)]
         w.keep = (lens_d, po, hist, smalls, caches)
         if which == "append":
-            w.name, w.kernel = "concat_kv_cache_f16_b8_q512_S1024", "isp::concat_kv_vec"
+            w.name, w.kernel = "concat_kv_cache_f16_b8_q512_S1024", "isp::concat_kv_vec<256>"
             w.bind(lib.isp_concat_kv_cache_f16,
                    [(smalls[j][0].data_ptr(), smalls[j][1].data_ptr(), caches[j][0].data_ptr(),
                      caches[j][1].data_ptr(), 0, lens_d.data_ptr(), hist.data_ptr(), batch, kvn, seq, max_seq, hs, st)
                     for j in range(R)])
         else:
-            w.name, w.kernel = "repeat_kv_cache_f16_b8_k512_S1024", "isp::repeat_kv_vec"
+            w.name, w.kernel = "repeat_kv_cache_f16_b8_k512_S1024", "isp::repeat_kv_vec<256>"
             w.bind(lib.isp_repeat_kv_cache_f16,
                    [(caches[j][0].data_ptr(), caches[j][1].data_ptr(), smalls[j][0].data_ptr(),
                      smalls[j][1].data_ptr(), 0, lens_d.data_ptr(), batch, hn, kvn, max_seq, seq, hs, st)
@@ -327,6 +368,8 @@ def make_workloads(torch, lib, stream_handle, rotate):
         ("rmsnorm_f32_16384x4096", lambda: norm("rmsnorm_f32_16384x4096", 16384, 4096, torch.float32, False)),
         ("embedding_f16_8192x4096_v32000", embedding),
         ("qkv_bias_rope_transpose_f16_b8_s512", qkv),
+        ("qkv_bias_rope_transpose_append_f16_b8_s512_S1024", lambda: qkv_append(True)),
+        ("qkv_bias_rope_transpose_then_concat_kv_f16_b8_s512_S1024", lambda: qkv_append(False)),
         ("swiglu_f16_prefill_8192x11008", lambda: swiglu(8192, "prefill")),
         ("swiglu_f16_decode_256x11008", lambda: swiglu(256, "decode")),
         ("transpose_remove_padding_f16_b8_s512", transpose_out),
@@ -477,15 +520,28 @@ def decode_sequence_record(torch, stream):
             stream.synchronize()
             return e0.elapsed_time(e1) * 1e3 / n
 
-        eager_us = timed(step, 200)
-        graph = torch.cuda.CUDAGraph()
-        graph.capture_begin()
-        step()
-        graph.capture_end()
-        stream.synchronize()
-        graph_us = timed(graph.replay, 200)
-    return {"workload": "decode_step_sequence_b16 (6 kernels)", "eager_us_per_step": eager_us,
-            "graph_replay_us_per_step": graph_us, "kernels_per_step": 6}
+        # the same step with bias + RoPE + append in one launch (the packed buffer then holds the whole batch)
+        qkv_b = h(batch, 96, 128)
+
+        def fused_step():
+            ops.fused_add_bias_residual_rmsnorm(residual, hidden, None, gamma, 1e-5)
+            ops.rope_decode_and_append(qkv_b, None, k_cache, v_cache, 0, hist, 101, 32, 128, 10000.0)
+            ops.repeat_kv_cache(k_cache, v_cache, ctx, 0, k_rep, v_rep)
+            ops.act(gate_up, act_out)
+            ops.rmsnorm(hidden, gamma, 1e-5)
+
+        out = {"workload": "decode_step_sequence_b16"}
+        for tag, fn, n_kernels in (("", step, 6), ("fused_", fused_step, 5)):
+            eager_us = timed(fn, 200)
+            graph = torch.cuda.CUDAGraph()
+            graph.capture_begin()
+            fn()
+            graph.capture_end()
+            stream.synchronize()
+            out[tag + "eager_us_per_step"] = eager_us
+            out[tag + "graph_replay_us_per_step"] = timed(graph.replay, 200)
+            out[tag + "kernels_per_step"] = n_kernels
+    return out
 
 
 # --------------------------------------------------------------------------- CPU baseline

@@ -138,6 +138,36 @@ int isp_qkv_bias_rope_transpose_f16(void* q, void* k, void* v, const void* qkv, 
                                     isp_stream_t stream);
 
 /*
+ * The same step with the KV-cache append fused in: besides (k, v non-NULL) or instead of (k, v both
+ * NULL) the padded k / v buffers, the k and v rows of token (b, s) are written to
+ *   cache[layer][b, head, history_length[b] + s, :]      when s < input_length[b]
+ * (rows that would fall outside [0, max_seq_len) are skipped), i.e. what launchConcatKVCache<T>
+ * (src/kernels/concat_past_kv.h:7-14, .cu:7-113) does in a second pass over k and v with
+ * cur_query_length = input_length.  The results are the bits of isp_qkv_bias_rope_transpose_*
+ * followed by isp_concat_kv_cache_*; one launch and one HBM pass less (with k, v NULL the k / v rows
+ * are written once instead of written, re-read and written again).
+ *   k_cache, v_cache [layers, batch, kv_head_num, max_seq_len, head_size] (base pointers).
+ * Extends launchAddFusedQKVBiasTransposeAndRoPE<T> (src/kernels/qkv_bias_and_RoPE.h:10-20); the
+ * reference has no fused form.
+ */
+int isp_qkv_bias_rope_transpose_append_f32(void* q, void* k, void* v, void* k_cache, void* v_cache,
+                                           int layer, int max_seq_len, const void* qkv,
+                                           const void* bias, const int32_t* padding_offset,
+                                           const int32_t* history_length,
+                                           const int32_t* input_length, int batch, int seq_len,
+                                           int token_num, int head_num, int kv_head_num,
+                                           int head_size, int rotary_embedding_dim,
+                                           float rotary_embedding_base, isp_stream_t stream);
+int isp_qkv_bias_rope_transpose_append_f16(void* q, void* k, void* v, void* k_cache, void* v_cache,
+                                           int layer, int max_seq_len, const void* qkv,
+                                           const void* bias, const int32_t* padding_offset,
+                                           const int32_t* history_length,
+                                           const int32_t* input_length, int batch, int seq_len,
+                                           int token_num, int head_num, int kv_head_num,
+                                           int head_size, int rotary_embedding_dim,
+                                           float rotary_embedding_base, isp_stream_t stream);
+
+/*
  * SwiGLU activation: out[t, i] = silu(in[t, 0, i]) * in[t, 1, i], silu(x) = x / (1 + exp(-x)).
  * Replaces launchAct<T> (src/kernels/act_kernel.h:8-9, .cu:18-71).
  *   in [tokens, 2, inter], out [tokens, inter].
@@ -155,6 +185,27 @@ int isp_rope_decode_f32(void* qkv, int batch, int head_num, int kv_head_num, int
                         int rotary_embedding_dim, float rotary_embedding_base, isp_stream_t stream);
 int isp_rope_decode_f16(void* qkv, int batch, int head_num, int kv_head_num, int head_size, int step,
                         int rotary_embedding_dim, float rotary_embedding_base, isp_stream_t stream);
+
+/*
+ * Fused decode step: QKV bias (may be NULL) + rotate-half RoPE at timestep step - 1, in place on the
+ * packed rows as isp_rope_decode_*, and the KV-cache append of the one new token per sequence:
+ *   k_cache[layer][b, head, history_length[b], :] = rotated k row,  v_cache[...] = v row
+ * (rows outside [0, max_seq_len) are skipped).  With the bias the v heads are updated in place too.
+ * One launch for launchRoPE<T> (src/kernels/qkv_bias_and_RoPE.cu:352-434) followed by
+ * launchConcatKVCache<T> with a one-token query (src/kernels/concat_past_kv.cu:7-113), whose results
+ * it reproduces bit for bit; each of the two is launch-bound alone.  The reference has no fused form
+ * outside its attention kernel (src/kernels/fused_decoder_self_attention.cu:162-200).
+ */
+int isp_rope_decode_append_f32(void* qkv, const void* bias, void* k_cache, void* v_cache, int layer,
+                               int max_seq_len, const int32_t* history_length, int batch,
+                               int head_num, int kv_head_num, int head_size, int step,
+                               int rotary_embedding_dim, float rotary_embedding_base,
+                               isp_stream_t stream);
+int isp_rope_decode_append_f16(void* qkv, const void* bias, void* k_cache, void* v_cache, int layer,
+                               int max_seq_len, const int32_t* history_length, int batch,
+                               int head_num, int kv_head_num, int head_size, int step,
+                               int rotary_embedding_dim, float rotary_embedding_base,
+                               isp_stream_t stream);
 
 /*
  * Transpose attention output and remove padding: dst[t, h, :] = src[b, h, s, :] with
@@ -240,7 +291,8 @@ typedef enum isp_tuning_knob {
                                         workgroup when a row needs fewer); 0 = automatic */
     ISP_TUNE_NORM_ORDER = 9,         /* 2 = streaming (each vector processed, and the residual stored, as it
                                         arrives); 0, 1 = read everything, then write everything (default) */
-    ISP_TUNE_COUNT = 10
+    ISP_TUNE_MOVER_BLOCK_THREADS = 10, /* KV append / broadcast: 256, 512 or 1024 threads per workgroup */
+    ISP_TUNE_COUNT = 11
 } isp_tuning_knob;
 int isp_tuning_set(int knob, int value);
 

@@ -13,7 +13,8 @@ ERR_LAUNCH = -4
 ERR_DEVICE = -5
 NORM_RESIDUAL_EXCLUDES_BIAS = 1
 (TUNE_NORM_WAVES_PER_ROW, TUNE_NORM_STORE, TUNE_SWIGLU_UNROLL, TUNE_SWIGLU_STORE, TUNE_EMBED_VARIANT,
- TUNE_EMBED_STORE, TUNE_QKV_STORE, TUNE_QKV_WAVES, TUNE_NORM_BLOCK_THREADS, TUNE_NORM_ORDER) = range(10)
+ TUNE_EMBED_STORE, TUNE_QKV_STORE, TUNE_QKV_WAVES, TUNE_NORM_BLOCK_THREADS, TUNE_NORM_ORDER,
+ TUNE_MOVER_BLOCK_THREADS) = range(11)
 
 _vp, _i, _f, _u = C.c_void_p, C.c_int, C.c_float, C.c_uint
 
@@ -32,10 +33,14 @@ SIGNATURES = {
     "isp_fused_add_bias_residual_rmsnorm_f16": (_i, [_vp, _vp, _vp, _vp, _f, _i, _i, _u, _vp]),
     "isp_qkv_bias_rope_transpose_f32": (_i, [_vp] * 8 + [_i] * 7 + [_f, _i, _i, _vp]),
     "isp_qkv_bias_rope_transpose_f16": (_i, [_vp] * 8 + [_i] * 7 + [_f, _i, _i, _vp]),
+    "isp_qkv_bias_rope_transpose_append_f32": (_i, [_vp] * 5 + [_i, _i] + [_vp] * 5 + [_i] * 7 + [_f, _vp]),
+    "isp_qkv_bias_rope_transpose_append_f16": (_i, [_vp] * 5 + [_i, _i] + [_vp] * 5 + [_i] * 7 + [_f, _vp]),
     "isp_swiglu_f32": (_i, [_vp, _vp, _i, _i, _vp]),
     "isp_swiglu_f16": (_i, [_vp, _vp, _i, _i, _vp]),
     "isp_rope_decode_f32": (_i, [_vp, _i, _i, _i, _i, _i, _i, _f, _vp]),
     "isp_rope_decode_f16": (_i, [_vp, _i, _i, _i, _i, _i, _i, _f, _vp]),
+    "isp_rope_decode_append_f32": (_i, [_vp] * 4 + [_i, _i, _vp] + [_i] * 6 + [_f, _vp]),
+    "isp_rope_decode_append_f16": (_i, [_vp] * 4 + [_i, _i, _vp] + [_i] * 6 + [_f, _vp]),
     "isp_transpose_remove_padding_f32": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "isp_transpose_remove_padding_f16": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "isp_concat_kv_cache_f32": (_i, [_vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _vp]),

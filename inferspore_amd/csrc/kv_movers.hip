@@ -81,8 +81,14 @@ __global__ __launch_bounds__(kBlock) void transpose_remove_padding_units(
 }
 
 // cache[b, h, history[b] + t, :] = src[b, h, t, :] for t < cur_len[b]; blockIdx.z selects k / v.
-// grid = (chunks of max_q_len*seg_vec vectors, batch * kv_heads, 2)
-__global__ __launch_bounds__(kBlock) void concat_kv_vec(
+// grid = (chunks of max_q_len*seg_vec vectors, batch * kv_heads, 2), a chunk being BLOCK vectors.
+// The grid has to cover max_q_len positions per sequence (the valid lengths live on the device), so the
+// workgroups behind a sequence's end leave at once but still cost their dispatch.  Larger workgroups
+// mean fewer of them, yet measured slower (batch 8 x 32 heads, lengths 256..512 of 512: 18.5 us with
+// 256 threads, 19.0 with 512, 19.6 with 1024; the broadcast 18.5 / 19.2 / 21.8), so 256 stays the
+// default and BLOCK a tuning knob (mover_block()).
+template <int BLOCK>
+__global__ __launch_bounds__(BLOCK) void concat_kv_vec(
     const char* __restrict__ k_src, const char* __restrict__ v_src, char* __restrict__ k_cache,
     char* __restrict__ v_cache, const int32_t* __restrict__ cur_query_length,
     const int32_t* __restrict__ history_length, int kv_head_num, int max_q_len, int max_seq_len,
@@ -92,7 +98,7 @@ __global__ __launch_bounds__(kBlock) void concat_kv_vec(
     char* cache = blockIdx.z == 0 ? k_cache : v_cache;
     const unsigned bh = blockIdx.y;
     const unsigned b = bh / kv_head_num;
-    const unsigned vi = blockIdx.x * kBlock + threadIdx.x;
+    const unsigned vi = blockIdx.x * BLOCK + threadIdx.x;
     if (vi >= (unsigned)max_q_len * seg_vec) return;
     unsigned t, c;
     sp.split(vi, t, c);
@@ -119,8 +125,9 @@ __global__ __launch_bounds__(kBlock) void concat_kv_units(
 }
 
 // dst[b, h, s, :] = cache[b, h / rep, s, :] for s < context_length[b]; blockIdx.z selects k / v.
-// grid = (chunks of max_k_len*seg_vec vectors, batch * heads, 2)
-__global__ __launch_bounds__(kBlock) void repeat_kv_vec(
+// grid = (chunks of max_k_len*seg_vec vectors, batch * heads, 2), a chunk being BLOCK vectors
+template <int BLOCK>
+__global__ __launch_bounds__(BLOCK) void repeat_kv_vec(
     const char* __restrict__ k_cache, const char* __restrict__ v_cache, char* __restrict__ k_dst,
     char* __restrict__ v_dst, const int32_t* __restrict__ context_length, int head_num,
     int kv_head_num, int max_seq_len, int max_k_len, SegSplit sp) {
@@ -129,7 +136,7 @@ __global__ __launch_bounds__(kBlock) void repeat_kv_vec(
     char* dst = blockIdx.z == 0 ? k_dst : v_dst;
     const unsigned bh = blockIdx.y;
     const unsigned b = bh / head_num, h = bh % head_num;
-    const unsigned vi = blockIdx.x * kBlock + threadIdx.x;
+    const unsigned vi = blockIdx.x * BLOCK + threadIdx.x;
     if (vi >= (unsigned)max_k_len * seg_vec) return;
     unsigned s, c;
     sp.split(vi, s, c);
@@ -155,6 +162,12 @@ __global__ __launch_bounds__(kBlock) void repeat_kv_units(
 }
 
 constexpr long long kMaxGridYZ = 65535;
+
+// Threads per workgroup of the cache movers: 256, 512 or 1024 (tuning knob, else the measured default).
+static int mover_block() {
+    const int knob = tuning(ISP_TUNE_MOVER_BLOCK_THREADS);
+    return (knob == 256 || knob == 512 || knob == 1024) ? knob : 256;
+}
 
 static int transpose_remove_padding(const void* src, const int32_t* padding_offset, void* dst,
                                     int batch, int head_num, int seq_len, int head_size,
@@ -213,9 +226,15 @@ static int concat_kv(const void* k_src, const void* v_src, void* k_cache, void* 
         const unsigned seg_vec = (unsigned)(seg / 16);
         const size_t row_vec = (size_t)max_q_len * seg_vec;
         if (row_vec > 0xffffffffull) return ISP_ERR_UNSUPPORTED;
-        dim3 grid((unsigned)((row_vec + kBlock - 1) / kBlock), (unsigned)(batch * kv_head_num), 2);
-        hipLaunchKernelGGL(concat_kv_vec, grid, dim3(kBlock), 0, s, ks, vs, kc, vc, cur_query_length,
-                           history_length, kv_head_num, max_q_len, max_seq_len, make_split(seg_vec));
+        const int blk = mover_block();
+        dim3 grid((unsigned)((row_vec + blk - 1) / blk), (unsigned)(batch * kv_head_num), 2);
+#define ISP_LAUNCH_CONCAT(B)                                                                       \
+    hipLaunchKernelGGL(concat_kv_vec<B>, grid, dim3(B), 0, s, ks, vs, kc, vc, cur_query_length,     \
+                       history_length, kv_head_num, max_q_len, max_seq_len, make_split(seg_vec))
+        if (blk == 1024) ISP_LAUNCH_CONCAT(1024);
+        else if (blk == 512) ISP_LAUNCH_CONCAT(512);
+        else ISP_LAUNCH_CONCAT(256);
+#undef ISP_LAUNCH_CONCAT
     } else {
         const dim3 grid((unsigned)max_q_len, (unsigned)(batch * kv_head_num), 2), block(kBlock);
 #define ISP_LAUNCH_UNITS(U)                                                                        \
@@ -256,9 +275,15 @@ static int repeat_kv(const void* k_cache, const void* v_cache, void* k_dst, void
         const unsigned seg_vec = (unsigned)(seg / 16);
         const size_t row_vec = (size_t)max_k_len * seg_vec;
         if (row_vec > 0xffffffffull) return ISP_ERR_UNSUPPORTED;
-        dim3 grid((unsigned)((row_vec + kBlock - 1) / kBlock), (unsigned)(batch * head_num), 2);
-        hipLaunchKernelGGL(repeat_kv_vec, grid, dim3(kBlock), 0, s, kc, vc, kd, vd, context_length,
-                           head_num, kv_head_num, max_seq_len, max_k_len, make_split(seg_vec));
+        const int blk = mover_block();
+        dim3 grid((unsigned)((row_vec + blk - 1) / blk), (unsigned)(batch * head_num), 2);
+#define ISP_LAUNCH_REPEAT(B)                                                                       \
+    hipLaunchKernelGGL(repeat_kv_vec<B>, grid, dim3(B), 0, s, kc, vc, kd, vd, context_length,       \
+                       head_num, kv_head_num, max_seq_len, max_k_len, make_split(seg_vec))
+        if (blk == 1024) ISP_LAUNCH_REPEAT(1024);
+        else if (blk == 512) ISP_LAUNCH_REPEAT(512);
+        else ISP_LAUNCH_REPEAT(256);
+#undef ISP_LAUNCH_REPEAT
     } else {
         const dim3 grid((unsigned)max_k_len, (unsigned)(batch * head_num), 2), block(kBlock);
 #define ISP_LAUNCH_UNITS(U)                                                                        \

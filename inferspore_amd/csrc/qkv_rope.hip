@@ -25,6 +25,9 @@
 //     read and write whole 128-byte lines of the 256-byte head rows and give identical bits;
 //   * stores are non-temporal write-through (q, k, v are consumed by a later kernel).
 #include <math.h>
+#include <stddef.h>
+
+#include <type_traits>
 
 #include "isp_common.h"
 
@@ -35,6 +38,26 @@ constexpr int kMaxHalfRot = 128;  // rotary_embedding_dim up to 256
 struct RopeDivisors {
     float div[kMaxHalfRot];
 };
+
+// Optional KV-cache append fused into the prefill step (what launchConcatKVCache does afterwards in
+// the reference, src/kernels/concat_past_kv.cu:7-73): the k and v rows of a token at position s of
+// sequence b also go to cache[b, head, history_length[b] + s, :] when s < input_length[b] and the row
+// lies inside the cache.  k_cache / v_cache point at the layer's slice; NULL = no append.
+template <typename T>
+struct KvAppend {
+    T* k_cache;
+    T* v_cache;
+    const int32_t* input_length;
+    int max_seq_len;
+};
+
+// Row of the cache a token at (b, s) is appended to, or -1.
+template <typename T>
+__device__ __forceinline__ long long append_row(const KvAppend<T>& ap, const int32_t* history_length, int b, int s) {
+    if (ap.k_cache == nullptr || s >= ap.input_length[b]) return -1;
+    const long long row = (long long)history_length[b] + s;
+    return (row >= 0 && row < ap.max_seq_len) ? row : -1;
+}
 
 // (cos, sin) of timestep / divisor: one correctly rounded division and the full-range sincosf, the
 // same two operations in every kernel of this file, so a decode step at `step` and a prefill token at
@@ -78,7 +101,7 @@ __global__ __launch_bounds__(kWave * WAVES) void qkv_rope_wave(
     T* __restrict__ q, T* __restrict__ k, T* __restrict__ v, const T* __restrict__ qkv,
     const T* __restrict__ bias, const int32_t* __restrict__ padding_offset,
     const int32_t* __restrict__ history_length, int batch, int seq_len, int head_num,
-    int kv_head_num, int half_rot, RopeDivisors tab) {
+    int kv_head_num, int half_rot, RopeDivisors tab, KvAppend<T> ap) {
     constexpr int VEC = Elem<T>::kVec;
     constexpr int HALF = HS / 2;
     constexpr int G = HALF / VEC;
@@ -153,15 +176,21 @@ __global__ __launch_bounds__(kWave * WAVES) void qkv_rope_wave(
             x1[e] += b1[e];
         }
     }
-    T* dst;
+    T* dst;        // row in the padded q / k / v buffer (k and v may be absent when appending)
+    T* cache = nullptr;  // row in the KV cache
     bool rotate = true;
     if (h < head_num) {
         dst = q + (((size_t)b * head_num + h) * seq_len + s) * HS;
-    } else if (h < head_num + kv_head_num) {
-        dst = k + (((size_t)b * kv_head_num + (h - head_num)) * seq_len + s) * HS;
     } else {
-        dst = v + (((size_t)b * kv_head_num + (h - head_num - kv_head_num)) * seq_len + s) * HS;
-        rotate = false;
+        const bool is_k = h < head_num + kv_head_num;
+        const int kvh = is_k ? h - head_num : h - head_num - kv_head_num;
+        T* plane = is_k ? k : v;
+        dst = plane ? plane + (((size_t)b * kv_head_num + kvh) * seq_len + s) * HS : nullptr;
+        rotate = is_k;
+        const long long row = append_row(ap, history_length, b, s);
+        if (row >= 0)
+            cache = (is_k ? ap.k_cache : ap.v_cache) +
+                    (((size_t)b * kv_head_num + kvh) * (size_t)ap.max_seq_len + (size_t)row) * HS;
     }
     float y0[VEC], y1[VEC];
 #pragma unroll
@@ -172,8 +201,15 @@ __global__ __launch_bounds__(kWave * WAVES) void qkv_rope_wave(
         y0[e] = r ? r0 : x0[e];
         y1[e] = r ? r1 : x1[e];
     }
-    store16_sel<ST>(dst + col, Elem<T>::pack(y0));
-    store16_sel<ST>(dst + HALF + col, Elem<T>::pack(y1));
+    const vec16 out0 = Elem<T>::pack(y0), out1 = Elem<T>::pack(y1);
+    if (dst) {
+        store16_sel<ST>(dst + col, out0);
+        store16_sel<ST>(dst + HALF + col, out1);
+    }
+    if (cache) {
+        store16_sel<ST>(cache + col, out0);
+        store16_sel<ST>(cache + HALF + col, out1);
+    }
 }
 
 // Unsigned division by a launch constant without the integer-divide expansion: q = floor(p / d) from
@@ -208,12 +244,15 @@ static FastDiv make_fastdiv(unsigned d) {
 // plane and sequence arithmetic is wave-uniform (scalar).  Same operations per element as
 // rotate_pair(), so the results are bit-identical to the other kernels of this file.  BIAS is a
 // template argument so that each variant has a fixed sequence of loads and the compiler's waits
-// are exact for it.
-template <int ST, bool BIAS>
+// are exact for it; so is APPEND (k and v rows also, or only, into the KV cache).
+// `tab` MUST stay the first parameter: first_argument_word() reads it at byte 0 of the argument
+// block (the launcher asserts its offset, and a test checks every coefficient through the ABI).
+template <int ST, bool BIAS, bool APPEND>
 __global__ __launch_bounds__(512) void qkv_rope_lean_f16(
     RopeDivisors tab, __half* q, __half* k, __half* v, const __half* qkv, const __half* bias,
     const int32_t* __restrict__ padding_offset, const int32_t* __restrict__ history_length,
-    unsigned positions, FastDiv seq, unsigned head_num, unsigned kv_head_num) {
+    unsigned positions, FastDiv seq, unsigned head_num, unsigned kv_head_num,
+    KvAppend<__half> ap) {
     constexpr unsigned ROW_BYTES = 256, GROUP = 32;
     const unsigned tid = threadIdx.x;
     const unsigned token = blockIdx.x;
@@ -248,9 +287,22 @@ __global__ __launch_bounds__(512) void qkv_rope_lean_f16(
     }
     char* dst = reinterpret_cast<char*>(plane) + (((size_t)b * plane_heads + h0) * seq.d + s) * ROW_BYTES;
     const unsigned lane_offset = (tid >> 4) * (seq.d * ROW_BYTES) + (tid & 15u) * 16u;  // head row, column
+    // the same group of rows in the KV cache (k and v groups only); all of it wave-uniform
+    char* cdst = nullptr;
+    unsigned cache_lane_offset = 0;
+    if (APPEND && first >= head_num) {
+        const long long row = append_row(ap, history_length, (int)b, (int)s);
+        if (row >= 0) {
+            cdst = reinterpret_cast<char*>(rotates ? ap.k_cache : ap.v_cache) +
+                   (((size_t)b * plane_heads + h0) * (size_t)ap.max_seq_len + (size_t)row) * ROW_BYTES;
+            cache_lane_offset = (tid >> 4) * ((unsigned)ap.max_seq_len * ROW_BYTES) + (tid & 15u) * 16u;
+        }
+        if (plane == nullptr && cdst == nullptr) return;  // nothing to write for this group
+    }
 
     if (!rotates && !BIAS) {  // v heads without bias: a plain move
-        store16_sel<ST>(dst + lane_offset, raw);
+        if (!APPEND || plane != nullptr) store16_sel<ST>(dst + lane_offset, raw);
+        if (APPEND && cdst != nullptr) store16_sel<ST>(cdst + cache_lane_offset, raw);
         return;
     }
     // the coefficient table first: the first wave evaluates it while every wave's loads are in flight
@@ -287,21 +339,37 @@ __global__ __launch_bounds__(512) void qkv_rope_lean_f16(
 #pragma unroll
         for (int e = 0; e < 8; e++) y[e] = x[e];
     }
-    store16_sel<ST>(dst + lane_offset, Elem<__half>::pack(y));
+    const vec16 packed = Elem<__half>::pack(y);
+    if (!APPEND || plane != nullptr) store16_sel<ST>(dst + lane_offset, packed);
+    if (APPEND && cdst != nullptr) store16_sel<ST>(cdst + cache_lane_offset, packed);
 }
+
+// first_argument_word() reads the divisor table at byte 0 of the kernel's argument block, where the
+// ABI puts the first explicit parameter: fail the build if that is ever something else.
+template <typename F>
+struct FirstParameter;
+template <typename A0, typename... A>
+struct FirstParameter<void (*)(A0, A...)> {
+    using type = A0;
+};
+static_assert(std::is_same<FirstParameter<decltype(&qkv_rope_lean_f16<kStorePlain, false, false>)>::type,
+                           RopeDivisors>::value &&
+                  offsetof(RopeDivisors, div) == 0,
+              "qkv_rope_lean_f16 must take the divisor table as its first parameter");
 
 // Any (even) head size and any alignment: one workgroup per token, one lane per rotation pair.
 template <typename T>
 __global__ __launch_bounds__(kBlock) void qkv_rope_generic(
     T* q, T* k, T* v, const T* qkv, const T* bias, const int32_t* padding_offset,
     const int32_t* history_length, int batch, int seq_len, int head_num, int kv_head_num,
-    int head_size, int half_rot, RopeDivisors tab) {
+    int head_size, int half_rot, RopeDivisors tab, KvAppend<T> ap) {
     const int token = blockIdx.x;
     const long long p = (long long)token + (long long)padding_offset[token];
     if (p < 0 || p >= (long long)batch * (long long)seq_len) return;
     const int b = (int)(p / seq_len);
     const int s = (int)(p % seq_len);
     const int timestep = history_length[b] + s;
+    const long long cache_row = append_row(ap, history_length, b, s);
     const int half = head_size / 2;
     const int qkv_heads = head_num + 2 * kv_head_num;
     const T* row = qkv + (size_t)token * (size_t)qkv_heads * head_size;
@@ -316,22 +384,34 @@ __global__ __launch_bounds__(kBlock) void qkv_rope_generic(
             x1 += Elem<T>::to_f32(bias[(size_t)h * head_size + half + d]);
         }
         T* dst;
+        T* cache = nullptr;
         bool rotate = d < half_rot;
         if (h < head_num) {
             dst = q + (((size_t)b * head_num + h) * seq_len + s) * head_size;
-        } else if (h < head_num + kv_head_num) {
-            dst = k + (((size_t)b * kv_head_num + (h - head_num)) * seq_len + s) * head_size;
         } else {
-            dst = v + (((size_t)b * kv_head_num + (h - head_num - kv_head_num)) * seq_len + s) * head_size;
-            rotate = false;
+            const bool is_k = h < head_num + kv_head_num;
+            const int kvh = is_k ? h - head_num : h - head_num - kv_head_num;
+            T* plane = is_k ? k : v;
+            dst = plane ? plane + (((size_t)b * kv_head_num + kvh) * seq_len + s) * head_size : nullptr;
+            rotate = rotate && is_k;
+            if (cache_row >= 0)
+                cache = (is_k ? ap.k_cache : ap.v_cache) +
+                        (((size_t)b * kv_head_num + kvh) * (size_t)ap.max_seq_len + (size_t)cache_row) * head_size;
         }
         float y0 = x0, y1 = x1;
         if (rotate) {
             const float2 coef = rope_coefficients(timestep, tab.div[d]);
             rotate_pair(coef.x, coef.y, x0, x1, y0, y1);
         }
-        dst[d] = Elem<T>::from_f32(y0);
-        dst[half + d] = Elem<T>::from_f32(y1);
+        const T o0 = Elem<T>::from_f32(y0), o1 = Elem<T>::from_f32(y1);
+        if (dst) {
+            dst[d] = o0;
+            dst[half + d] = o1;
+        }
+        if (cache) {
+            cache[d] = o0;
+            cache[half + d] = o1;
+        }
     }
 }
 
@@ -341,10 +421,26 @@ __global__ __launch_bounds__(kBlock) void qkv_rope_generic(
 // one row, evaluates the 64 (cos, sin) pairs once and shares them through wave-private LDS.
 // Each k head is rotated once (the reference rotates k head q / (head_num / kv_head_num) from every q
 // block, which only coincides with this when kv_head_num == head_num, the one case it accepts).
+//
+// The same kernels also run the fused decode step (DecodeExtras): the QKV bias added first, and the
+// rotated k row and the v row of sequence b appended to cache[b, head, history_length[b], :] -- what
+// launchConcatKVCache does for a one-token query (src/kernels/concat_past_kv.cu:7-73) -- so that a
+// decode step needs one launch instead of three launch-bound ones.  With all extras absent only the
+// q and k heads are touched, exactly as before.
+template <typename T>
+struct DecodeExtras {
+    const T* bias;                   // [(head_num + 2 kv_head_num) * head_size] or NULL
+    T* k_cache;                      // layer slice [batch, kv_head_num, max_seq_len, head_size] or NULL
+    T* v_cache;
+    const int32_t* history_length;   // [batch]; read only when appending
+    int max_seq_len;
+};
+
 template <typename T, int HS>
 __global__ __launch_bounds__(kBlock) void rope_decode_wave(T* __restrict__ qkv, int head_num,
                                                            int kv_head_num, int timestep,
-                                                           int half_rot, RopeDivisors tab) {
+                                                           int half_rot, RopeDivisors tab,
+                                                           DecodeExtras<T> ex) {
     constexpr int VEC = Elem<T>::kVec;
     constexpr int HALF = HS / 2;
     constexpr int G = HALF / VEC;
@@ -355,15 +451,22 @@ __global__ __launch_bounds__(kBlock) void rope_decode_wave(T* __restrict__ qkv, 
     const int g = lane % G;
     const int slot = lane / G;
     const int rotated_heads = head_num + kv_head_num;
+    const bool extras = ex.bias != nullptr || ex.k_cache != nullptr;
+    const int covered = extras ? rotated_heads + kv_head_num : rotated_heads;  // v heads only with extras
     const int wave_first = ((int)blockIdx.y * WAVES + wave) * HEADS_PER_WAVE;
-    if (wave_first >= rotated_heads) return;  // wave-uniform
+    if (wave_first >= covered) return;  // wave-uniform
     const int h = wave_first + slot;
-    const bool live = h < rotated_heads;
-    T* p = qkv + ((size_t)blockIdx.x * (size_t)(head_num + 2 * kv_head_num) + (live ? h : 0)) * HS + g * VEC;
-    vec16 lo, hi;
+    const bool live = h < covered;
+    const int b = (int)blockIdx.x;
+    T* p = qkv + ((size_t)b * (size_t)(head_num + 2 * kv_head_num) + (live ? h : 0)) * HS + g * VEC;
+    vec16 lo, hi, blo, bhi;
     if (live) {
         lo = load16(p);
         hi = load16(p + HALF);
+        if (ex.bias) {
+            blo = load16(ex.bias + (size_t)h * HS + g * VEC);
+            bhi = load16(ex.bias + (size_t)h * HS + HALF + g * VEC);
+        }
     }
     __shared__ float2 cs[WAVES][HALF];
     if (lane < HALF) {
@@ -375,38 +478,91 @@ __global__ __launch_bounds__(kBlock) void rope_decode_wave(T* __restrict__ qkv, 
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     if (!live) return;
+    const bool is_v = h >= rotated_heads;
     float x0[VEC], x1[VEC], y0[VEC], y1[VEC];
     Elem<T>::unpack(lo, x0);
     Elem<T>::unpack(hi, x1);
+    if (ex.bias) {
+        float b0[VEC], b1[VEC];
+        Elem<T>::unpack(blo, b0);
+        Elem<T>::unpack(bhi, b1);
+#pragma unroll
+        for (int e = 0; e < VEC; e++) {
+            x0[e] += b0[e];
+            x1[e] += b1[e];
+        }
+    }
 #pragma unroll
     for (int e = 0; e < VEC; e++) {
         const float2 t = cs[wave][g * VEC + e];
-        const bool r = (g * VEC + e) < half_rot;
+        const bool r = !is_v && (g * VEC + e) < half_rot;
         float r0, r1;
         rotate_pair(t.x, t.y, x0[e], x1[e], r0, r1);
         y0[e] = r ? r0 : x0[e];
         y1[e] = r ? r1 : x1[e];
     }
-    store16(p, Elem<T>::pack(y0));
-    store16(p + HALF, Elem<T>::pack(y1));
+    const vec16 out0 = Elem<T>::pack(y0), out1 = Elem<T>::pack(y1);
+    if (!is_v || ex.bias) {  // a v row without bias is unchanged
+        store16(p, out0);
+        store16(p + HALF, out1);
+    }
+    if (ex.k_cache && h >= head_num) {
+        const long long row = ex.history_length[b];
+        if (row >= 0 && row < ex.max_seq_len) {
+            const int kvh = is_v ? h - rotated_heads : h - head_num;
+            T* c = (is_v ? ex.v_cache : ex.k_cache) +
+                   (((size_t)b * kv_head_num + kvh) * (size_t)ex.max_seq_len + (size_t)row) * HS + g * VEC;
+            store16(c, out0);
+            store16(c + HALF, out1);
+        }
+    }
 }
 
 template <typename T>
 __global__ __launch_bounds__(kBlock) void rope_decode_generic(T* qkv, int head_num, int kv_head_num,
                                                               int head_size, int timestep,
-                                                              int half_rot, RopeDivisors tab) {
+                                                              int half_rot, RopeDivisors tab,
+                                                              DecodeExtras<T> ex) {
     const int half = head_size / 2;
-    T* row = qkv + (size_t)blockIdx.x * (size_t)(head_num + 2 * kv_head_num) * head_size;
-    const int pairs = (head_num + kv_head_num) * half_rot;
+    const int b = (int)blockIdx.x;
+    T* row = qkv + (size_t)b * (size_t)(head_num + 2 * kv_head_num) * head_size;
+    const int rotated_heads = head_num + kv_head_num;
+    const bool extras = ex.bias != nullptr || ex.k_cache != nullptr;
+    const int covered = extras ? rotated_heads + kv_head_num : rotated_heads;
+    // without extras only the rotated pairs are touched; with them every pair of every covered head
+    const int per_head = extras ? half : half_rot;
+    const int pairs = covered * per_head;
+    long long cache_row = -1;
+    if (ex.k_cache) {
+        cache_row = ex.history_length[b];
+        if (cache_row < 0 || cache_row >= ex.max_seq_len) cache_row = -1;
+    }
     for (int i = threadIdx.x; i < pairs; i += kBlock) {
-        const int h = i / half_rot, d = i % half_rot;
+        const int h = i / per_head, d = i % per_head;
+        const bool is_v = h >= rotated_heads;
         T* p = row + (size_t)h * head_size + d;
-        const float x0 = Elem<T>::to_f32(p[0]), x1 = Elem<T>::to_f32(p[half]);
-        float y0, y1;
-        const float2 coef = rope_coefficients(timestep, tab.div[d]);
-        rotate_pair(coef.x, coef.y, x0, x1, y0, y1);
-        p[0] = Elem<T>::from_f32(y0);
-        p[half] = Elem<T>::from_f32(y1);
+        float x0 = Elem<T>::to_f32(p[0]), x1 = Elem<T>::to_f32(p[half]);
+        if (ex.bias) {
+            x0 += Elem<T>::to_f32(ex.bias[(size_t)h * head_size + d]);
+            x1 += Elem<T>::to_f32(ex.bias[(size_t)h * head_size + half + d]);
+        }
+        float y0 = x0, y1 = x1;
+        if (!is_v && d < half_rot) {
+            const float2 coef = rope_coefficients(timestep, tab.div[d]);
+            rotate_pair(coef.x, coef.y, x0, x1, y0, y1);
+        }
+        const T o0 = Elem<T>::from_f32(y0), o1 = Elem<T>::from_f32(y1);
+        if (!is_v || ex.bias) {
+            p[0] = o0;
+            p[half] = o1;
+        }
+        if (cache_row >= 0 && h >= head_num) {
+            const int kvh = is_v ? h - rotated_heads : h - head_num;
+            T* c = (is_v ? ex.v_cache : ex.k_cache) +
+                   (((size_t)b * kv_head_num + kvh) * (size_t)ex.max_seq_len + (size_t)cache_row) * head_size + d;
+            c[0] = o0;
+            c[half] = o1;
+        }
     }
 }
 
@@ -427,43 +583,66 @@ static void fill_divisors(RopeDivisors& tab, int rot, float base) {
     tab = cached;
 }
 
+// bias_ / caches NULL: plain launchRoPE.  Otherwise the fused decode step (see DecodeExtras).
 template <typename T>
 static int rope_decode(void* qkv_, int batch, int head_num, int kv_head_num, int head_size, int step,
-                       int rot, float base, hipStream_t s) {
-    if (batch < 0 || head_num < 0 || kv_head_num < 0 || head_size < 0 || rot < 0) return ISP_ERR_BAD_SHAPE;
-    if (batch == 0 || head_size == 0 || head_num + kv_head_num == 0 || rot == 0) return ISP_OK;
+                       int rot, float base, hipStream_t s, const void* bias_ = nullptr,
+                       void* k_cache_ = nullptr, void* v_cache_ = nullptr, int layer = 0,
+                       int max_seq_len = 0, const int32_t* history_length = nullptr) {
+    if (batch < 0 || head_num < 0 || kv_head_num < 0 || head_size < 0 || rot < 0 || layer < 0 || max_seq_len < 0)
+        return ISP_ERR_BAD_SHAPE;
+    const bool append = k_cache_ != nullptr || v_cache_ != nullptr;
+    const bool extras = append || bias_ != nullptr;
+    if (batch == 0 || head_size == 0 || head_num + kv_head_num == 0) return ISP_OK;
+    if (rot == 0 && !extras) return ISP_OK;
     if (head_size % 2 != 0 || rot % 2 != 0 || rot > head_size) return ISP_ERR_BAD_SHAPE;
     if (rot / 2 > kMaxHalfRot) return ISP_ERR_UNSUPPORTED;
     ISP_REQUIRE_PTR(qkv_);
     T* qkv = static_cast<T*>(qkv_);
+    DecodeExtras<T> ex = {static_cast<const T*>(bias_), nullptr, nullptr, history_length, max_seq_len};
+    if (append && kv_head_num > 0) {
+        ISP_REQUIRE_PTR(k_cache_);
+        ISP_REQUIRE_PTR(v_cache_);
+        ISP_REQUIRE_PTR(history_length);
+        const size_t layer_elems = (size_t)layer * batch * kv_head_num * max_seq_len * head_size;  // concat_past_kv.cu:89
+        ex.k_cache = static_cast<T*>(k_cache_) + layer_elems;
+        ex.v_cache = static_cast<T*>(v_cache_) + layer_elems;
+    }
     RopeDivisors tab;
     fill_divisors(tab, rot, base);
     const int timestep = step - 1;  // qkv_bias_and_RoPE.cu:380
     const int half_rot = rot / 2;
+    const int covered = head_num + kv_head_num + ((ex.bias || ex.k_cache) ? kv_head_num : 0);
     dim3 block(kBlock);
-    if (aligned16(qkv) && (head_size == 128 || head_size == 64) && head_num + kv_head_num <= 65535) {
+    const bool vec_ok = aligned16(qkv) && aligned16(ex.bias) && aligned16(ex.k_cache) && aligned16(ex.v_cache);
+    if (vec_ok && (head_size == 128 || head_size == 64) && covered <= 65535) {
         const int hpb = (kWave / ((head_size / 2) / Elem<T>::kVec)) * (kBlock / kWave);
-        dim3 grid((unsigned)batch, (unsigned)((head_num + kv_head_num + hpb - 1) / hpb));
+        dim3 grid((unsigned)batch, (unsigned)((covered + hpb - 1) / hpb));
         if (head_size == 128)
             hipLaunchKernelGGL((rope_decode_wave<T, 128>), grid, block, 0, s, qkv, head_num, kv_head_num,
-                               timestep, half_rot, tab);
+                               timestep, half_rot, tab, ex);
         else
             hipLaunchKernelGGL((rope_decode_wave<T, 64>), grid, block, 0, s, qkv, head_num, kv_head_num,
-                               timestep, half_rot, tab);
+                               timestep, half_rot, tab, ex);
     } else {
         hipLaunchKernelGGL((rope_decode_generic<T>), dim3((unsigned)batch), block, 0, s, qkv, head_num,
-                           kv_head_num, head_size, timestep, half_rot, tab);
+                           kv_head_num, head_size, timestep, half_rot, tab, ex);
     }
     return note_launch(hipGetLastError());
 }
 
+// `append`: also (k_ / v_ non-NULL) or only (k_ / v_ NULL) write the k and v rows into the KV cache
+// [layers, batch, kv_head_num, max_seq_len, head_size] at layer `layer`.
 template <typename T>
 static int qkv_rope(void* q_, void* k_, void* v_, const void* qkv_, const void* bias_,
                     const int32_t* padding_offset, const int32_t* history_length,
                     const int32_t* input_length, int batch, int seq_len, int token_num,
                     int head_num, int kv_head_num, int head_size, int rot, float base,
-                    hipStream_t s) {
-    (void)input_length;  // read by the reference kernel, result unused (qkv_bias_and_RoPE.cu:161)
+                    hipStream_t s, bool append = false, void* k_cache_ = nullptr,
+                    void* v_cache_ = nullptr, int layer = 0, int max_seq_len = 0) {
+    // without `append`, input_length is read by the reference kernel but its value is unused
+    // (qkv_bias_and_RoPE.cu:161)
+    if (append && (layer < 0 || max_seq_len < 0)) return ISP_ERR_BAD_SHAPE;
     if (batch < 0 || seq_len < 0 || token_num < 0 || head_num < 0 || kv_head_num < 0 ||
         head_size < 0 || rot < 0)
         return ISP_ERR_BAD_SHAPE;
@@ -477,22 +656,33 @@ static int qkv_rope(void* q_, void* k_, void* v_, const void* qkv_, const void* 
     ISP_REQUIRE_PTR(padding_offset);
     ISP_REQUIRE_PTR(history_length);
     if (head_num > 0) ISP_REQUIRE_PTR(q_);
-    if (kv_head_num > 0) {
+    if (kv_head_num > 0 && !append) {
         ISP_REQUIRE_PTR(k_);
         ISP_REQUIRE_PTR(v_);
     }
+    if ((k_ == nullptr) != (v_ == nullptr)) return ISP_ERR_NULL_POINTER;
     T* q = static_cast<T*>(q_);
     T* k = static_cast<T*>(k_);
     T* v = static_cast<T*>(v_);
     const T* qkv = static_cast<const T*>(qkv_);
     const T* bias = static_cast<const T*>(bias_);
+    KvAppend<T> ap = {nullptr, nullptr, input_length, max_seq_len};
+    if (append && kv_head_num > 0) {
+        ISP_REQUIRE_PTR(k_cache_);
+        ISP_REQUIRE_PTR(v_cache_);
+        ISP_REQUIRE_PTR(input_length);
+        // layer offset as in launchConcatKVCache (concat_past_kv.cu:89)
+        const size_t layer_elems = (size_t)layer * batch * kv_head_num * max_seq_len * head_size;
+        ap.k_cache = static_cast<T*>(k_cache_) + layer_elems;
+        ap.v_cache = static_cast<T*>(v_cache_) + layer_elems;
+    }
 
     RopeDivisors tab;
     const int half_rot = rot / 2;
     fill_divisors(tab, rot, base);
 
     const bool vec_ok = aligned16(q) && aligned16(k) && aligned16(v) && aligned16(qkv) &&
-                        (!bias || aligned16(bias));
+                        (!bias || aligned16(bias)) && aligned16(ap.k_cache) && aligned16(ap.v_cache);
     dim3 grid((unsigned)token_num), block(kBlock);
     hipError_t e;
     const int kind = store_kind(tuning(ISP_TUNE_QKV_STORE), kStoreThrough);
@@ -504,7 +694,7 @@ static int qkv_rope(void* q_, void* k_, void* v_, const void* qkv_, const void* 
         dim3 g2((unsigned)token_num, (unsigned)((head_num + 2 * kv_head_num + HPB - 1) / HPB));    \
         hipLaunchKernelGGL((qkv_rope_wave<T, HS, K, W>), g2, dim3(kWave * W), 0, s, q, k, v, qkv,   \
                            bias, padding_offset, history_length, batch, seq_len, head_num,         \
-                           kv_head_num, half_rot, tab);                                            \
+                           kv_head_num, half_rot, tab, ap);                                        \
     } while (0)
 #define ISP_QKV_LAUNCH_K(HS, W)                                                                    \
     do {                                                                                           \
@@ -526,6 +716,7 @@ static int qkv_rope(void* q_, void* k_, void* v_, const void* qkv_, const void* 
                          head_num % 32 == 0 && kv_head_num % 32 == 0 &&
                          (head_num + 2 * kv_head_num) / 32 <= 65535 &&
                          (unsigned long long)seq_len * 256ull * 32ull <= 0xffffffffull &&
+                         (unsigned long long)max_seq_len * 256ull * 32ull <= 0xffffffffull &&
                          (unsigned long long)batch * (unsigned long long)seq_len <= 0x7fffffffull &&
                          (waves_knob <= 0 || waves_knob >= 8);
     if (lean_ok) {
@@ -537,20 +728,24 @@ static int qkv_rope(void* q_, void* k_, void* v_, const void* qkv_, const void* 
         __half* vh = reinterpret_cast<__half*>(v);
         const __half* xh = reinterpret_cast<const __half*>(qkv);
         const __half* bh = reinterpret_cast<const __half*>(bias);
+        KvAppend<__half> aph = {reinterpret_cast<__half*>(ap.k_cache), reinterpret_cast<__half*>(ap.v_cache),
+                                ap.input_length, ap.max_seq_len};
+        const bool with_append = aph.k_cache != nullptr;
+#define ISP_QKV_LEAN_2(K, B, A)                                                                    \
+    hipLaunchKernelGGL((qkv_rope_lean_f16<K, B, A>), g2, dim3(512), 0, s, tab, qh, kh, vh, xh, bh,  \
+                       padding_offset, history_length, positions, fd, (unsigned)head_num,          \
+                       (unsigned)kv_head_num, aph)
 #define ISP_QKV_LEAN(K)                                                                            \
     do {                                                                                           \
-        if (bh)                                                                                    \
-            hipLaunchKernelGGL((qkv_rope_lean_f16<K, true>), g2, dim3(512), 0, s, tab, qh, kh, vh,  \
-                               xh, bh, padding_offset, history_length, positions, fd,              \
-                               (unsigned)head_num, (unsigned)kv_head_num);                         \
-        else                                                                                       \
-            hipLaunchKernelGGL((qkv_rope_lean_f16<K, false>), g2, dim3(512), 0, s, tab, qh, kh, vh, \
-                               xh, bh, padding_offset, history_length, positions, fd,              \
-                               (unsigned)head_num, (unsigned)kv_head_num);                         \
+        if (bh && with_append) ISP_QKV_LEAN_2(K, true, true);                                      \
+        else if (bh) ISP_QKV_LEAN_2(K, true, false);                                               \
+        else if (with_append) ISP_QKV_LEAN_2(K, false, true);                                      \
+        else ISP_QKV_LEAN_2(K, false, false);                                                      \
     } while (0)
         if (kind == kStoreThrough) ISP_QKV_LEAN(kStoreThrough);
         else if (kind == kStoreStream) ISP_QKV_LEAN(kStoreStream);
         else ISP_QKV_LEAN(kStorePlain);
+#undef ISP_QKV_LEAN_2
 #undef ISP_QKV_LEAN
         e = hipGetLastError();
     } else if (vec_ok && head_size == 128 && head_num + 2 * kv_head_num <= head_groups_max) {
@@ -562,7 +757,7 @@ static int qkv_rope(void* q_, void* k_, void* v_, const void* qkv_, const void* 
     } else {
         hipLaunchKernelGGL((qkv_rope_generic<T>), grid, block, 0, s, q, k, v, qkv, bias,
                            padding_offset, history_length, batch, seq_len, head_num, kv_head_num,
-                           head_size, half_rot, tab);
+                           head_size, half_rot, tab, ap);
         e = hipGetLastError();
     }
     return note_launch(e);
@@ -600,6 +795,58 @@ int isp_qkv_bias_rope_transpose_f16(void* q, void* k, void* v, const void* qkv, 
                                  batch, seq_len, token_num, head_num, kv_head_num, head_size,
                                  rotary_embedding_dim, rotary_embedding_base,
                                  static_cast<hipStream_t>(stream));
+}
+
+int isp_qkv_bias_rope_transpose_append_f32(void* q, void* k, void* v, void* k_cache, void* v_cache,
+                                           int layer, int max_seq_len, const void* qkv,
+                                           const void* bias, const int32_t* padding_offset,
+                                           const int32_t* history_length,
+                                           const int32_t* input_length, int batch, int seq_len,
+                                           int token_num, int head_num, int kv_head_num,
+                                           int head_size, int rotary_embedding_dim,
+                                           float rotary_embedding_base, isp_stream_t stream) {
+    return isp::qkv_rope<float>(q, k, v, qkv, bias, padding_offset, history_length, input_length,
+                                batch, seq_len, token_num, head_num, kv_head_num, head_size,
+                                rotary_embedding_dim, rotary_embedding_base,
+                                static_cast<hipStream_t>(stream), true, k_cache, v_cache, layer,
+                                max_seq_len);
+}
+
+int isp_qkv_bias_rope_transpose_append_f16(void* q, void* k, void* v, void* k_cache, void* v_cache,
+                                           int layer, int max_seq_len, const void* qkv,
+                                           const void* bias, const int32_t* padding_offset,
+                                           const int32_t* history_length,
+                                           const int32_t* input_length, int batch, int seq_len,
+                                           int token_num, int head_num, int kv_head_num,
+                                           int head_size, int rotary_embedding_dim,
+                                           float rotary_embedding_base, isp_stream_t stream) {
+    return isp::qkv_rope<__half>(q, k, v, qkv, bias, padding_offset, history_length, input_length,
+                                 batch, seq_len, token_num, head_num, kv_head_num, head_size,
+                                 rotary_embedding_dim, rotary_embedding_base,
+                                 static_cast<hipStream_t>(stream), true, k_cache, v_cache, layer,
+                                 max_seq_len);
+}
+
+int isp_rope_decode_append_f32(void* qkv, const void* bias, void* k_cache, void* v_cache, int layer,
+                               int max_seq_len, const int32_t* history_length, int batch,
+                               int head_num, int kv_head_num, int head_size, int step,
+                               int rotary_embedding_dim, float rotary_embedding_base,
+                               isp_stream_t stream) {
+    return isp::rope_decode<float>(qkv, batch, head_num, kv_head_num, head_size, step,
+                                   rotary_embedding_dim, rotary_embedding_base,
+                                   static_cast<hipStream_t>(stream), bias, k_cache, v_cache, layer,
+                                   max_seq_len, history_length);
+}
+
+int isp_rope_decode_append_f16(void* qkv, const void* bias, void* k_cache, void* v_cache, int layer,
+                               int max_seq_len, const int32_t* history_length, int batch,
+                               int head_num, int kv_head_num, int head_size, int step,
+                               int rotary_embedding_dim, float rotary_embedding_base,
+                               isp_stream_t stream) {
+    return isp::rope_decode<__half>(qkv, batch, head_num, kv_head_num, head_size, step,
+                                    rotary_embedding_dim, rotary_embedding_base,
+                                    static_cast<hipStream_t>(stream), bias, k_cache, v_cache, layer,
+                                    max_seq_len, history_length);
 }
 
 int isp_rope_decode_f32(void* qkv, int batch, int head_num, int kv_head_num, int head_size, int step,

@@ -145,3 +145,28 @@ def test_calibration_copy(isp):
         dst = torch.zeros(nbytes + 16, dtype=torch.uint8, device="cuda")
         capi.check(lib.isp_calibration_copy(dst.data_ptr(), src.data_ptr(), nbytes, st), "isp_calibration_copy")
         assert torch.equal(dst[:nbytes], src) and int(dst[nbytes:].sum()) == 0
+
+
+def test_kv_movers_every_workgroup_size(isp):
+    from inferspore_amd import capi
+    batch, kvn, hn, q_len, max_seq, hs = 3, 2, 4, 70, 96, 128
+    g = torch.Generator(device="cuda").manual_seed(3)
+    k_src = torch.randn((batch, kvn, q_len, hs), device="cuda", generator=g).half()
+    v_src = torch.randn((batch, kvn, q_len, hs), device="cuda", generator=g).half()
+    lens = torch.tensor([70, 1, 33], dtype=torch.int32, device="cuda")
+    hist = torch.tensor([5, 0, 26], dtype=torch.int32, device="cuda")
+
+    def run():
+        kc = torch.full((1, batch, kvn, max_seq, hs), -2.0, dtype=torch.float16, device="cuda")
+        vc = kc.clone()
+        isp.concat_kv_cache(k_src, v_src, 0, lens, hist, kc, vc)
+        kd = torch.full((batch, hn, max_seq, hs), -3.0, dtype=torch.float16, device="cuda")
+        vd = kd.clone()
+        isp.repeat_kv_cache(kc, vc, lens + hist, 0, kd, vd)
+        return [t.cpu().numpy() for t in (kc, vc, kd, vd)]
+
+    base = run()
+    for block in (256, 512, 1024):
+        say("kv movers with %d-thread workgroups" % block)
+        got = with_knobs({capi.TUNE_MOVER_BLOCK_THREADS: block}, run)
+        assert all(np.array_equal(a, b) for a, b in zip(got, base))
