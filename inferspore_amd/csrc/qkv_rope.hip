@@ -91,6 +91,27 @@ __device__ __forceinline__ void rotate_pair(float c, float sn, float x0, float x
     y1 = __fmaf_rn(c, x1, sn * x0);
 }
 
+// Unsigned division by a launch constant without the integer-divide expansion: q = floor(p / d) from
+// one multiply-high and one correction step (exact for every 32-bit p).
+struct FastDiv {
+    unsigned d, m;  // m = floor(2^32 / d), saturated for d = 1
+    __device__ __forceinline__ void divmod(unsigned p, unsigned& q, unsigned& r) const {
+        q = __umulhi(p, m);
+        r = p - q * d;
+        if (r >= d) {
+            q++;
+            r -= d;
+        }
+    }
+};
+
+static FastDiv make_fastdiv(unsigned d) {
+    FastDiv f;
+    f.d = d;
+    f.m = d <= 1 ? 0xffffffffu : (unsigned)(0x100000000ull / d);
+    return f;
+}
+
 // A wave owns kWave / G consecutive heads of one token (one head-half pair per lane: two loads and
 // two stores).  The first wave of a workgroup evaluates the token's (cos, sin) pairs (lane d
 // evaluates pair d) and shares them through LDS behind one barrier (measured 3 % faster than every
@@ -100,11 +121,12 @@ template <typename T, int HS, int ST, int WAVES>
 __global__ __launch_bounds__(kWave * WAVES) void qkv_rope_wave(
     T* __restrict__ q, T* __restrict__ k, T* __restrict__ v, const T* __restrict__ qkv,
     const T* __restrict__ bias, const int32_t* __restrict__ padding_offset,
-    const int32_t* __restrict__ history_length, int batch, int seq_len, int head_num,
+    const int32_t* __restrict__ history_length, unsigned positions, FastDiv seq, int head_num,
     int kv_head_num, int half_rot, RopeDivisors tab, KvAppend<T> ap) {
     constexpr int VEC = Elem<T>::kVec;
     constexpr int HALF = HS / 2;
     constexpr int G = HALF / VEC;
+    const int seq_len = (int)seq.d;
     static_assert(HALF % VEC == 0 && kWave % G == 0 && HALF <= kWave, "unsupported head size");
     constexpr int HEADS_PER_WAVE = kWave / G;
 
@@ -136,10 +158,12 @@ __global__ __launch_bounds__(kWave * WAVES) void qkv_rope_wave(
             bhi = load16(bias + (size_t)h * HS + HALF + col);
         }
     }
+    // wave-uniform: scalar arithmetic, the division by seq_len as a multiply-high
     const long long p = (long long)token + (long long)padding_offset[token];
-    if (p < 0 || p >= (long long)batch * (long long)seq_len) return;  // wave-uniform
-    const int b = (int)(p / seq_len);
-    const int s = (int)(p % seq_len);
+    if (p < 0 || p >= (long long)positions) return;
+    unsigned ub, us;
+    seq.divmod((unsigned)p, ub, us);
+    const int b = (int)ub, s = (int)us;
 
     float c[VEC], sn[VEC];
 #pragma unroll
@@ -212,25 +236,108 @@ __global__ __launch_bounds__(kWave * WAVES) void qkv_rope_wave(
     }
 }
 
-// Unsigned division by a launch constant without the integer-divide expansion: q = floor(p / d) from
-// one multiply-high and one correction step (exact for every 32-bit p).
-struct FastDiv {
-    unsigned d, m;  // m = floor(2^32 / d), saturated for d = 1
-    __device__ __forceinline__ void divmod(unsigned p, unsigned& q, unsigned& r) const {
-        q = __umulhi(p, m);
-        r = p - q * d;
-        if (r >= d) {
-            q++;
-            r -= d;
+// fp16 heads of 64 elements: a head row is 128 bytes = 8 lanes x 16 bytes, so with one vector per lane
+// every load and store instruction of a wave covers 8 whole rows (the general kernel above, whose
+// lanes own a half-row vector and its partner 64 bytes further on, moves half rows per instruction
+// at this head size: 51-57 % of the peak bandwidth against 57-65 % here).  The rotation partner
+// d +- 32 sits 4 lanes away: two DPP row rotations, each enabled for the lane banks it serves, fetch
+// it in the VALU.  Same arithmetic per element as rotate_pair(): bit-identical to the other kernels.
+// (Measured and not kept: two consecutive tokens per wave in neighbouring lane groups, so that stores
+// cover 256 contiguous bytes as with 128-element heads -- 6-10 % slower.)
+// grid = (tokens, groups of 8 * WAVES heads).
+template <int ST, int WAVES>
+__global__ __launch_bounds__(kWave * WAVES) void qkv_rope_rows64_f16(
+    __half* __restrict__ q, __half* __restrict__ k, __half* __restrict__ v,
+    const __half* __restrict__ qkv, const __half* __restrict__ bias,
+    const int32_t* __restrict__ padding_offset, const int32_t* __restrict__ history_length,
+    unsigned positions, FastDiv seq, int head_num, int kv_head_num, int half_rot, RopeDivisors tab,
+    KvAppend<__half> ap) {
+    constexpr int HS = 64, HALF = 32, VEC = 8, LANES_PER_ROW = 8, HEADS_PER_WAVE = kWave / LANES_PER_ROW;
+    const int seq_len = (int)seq.d;
+    const int lane = threadIdx.x % kWave;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const int token = (int)blockIdx.x;
+    const int g = lane % LANES_PER_ROW;   // column group: elements 8 g .. 8 g + 7 of the row
+    const int slot = lane / LANES_PER_ROW;
+    const int qkv_heads = head_num + 2 * kv_head_num;
+    const int h = ((int)blockIdx.y * WAVES + wave) * HEADS_PER_WAVE + slot;
+    const bool live = h < qkv_heads;
+    const int col = g * VEC;
+    vec16 raw, braw;
+    if (live) {
+        raw = load16_stream(qkv + ((size_t)token * (size_t)qkv_heads + h) * HS + col);
+        if (bias) braw = load16(bias + (size_t)h * HS + col);
+    }
+    const long long p = (long long)token + (long long)padding_offset[token];
+    if (p < 0 || p >= (long long)positions) return;  // workgroup-uniform
+    unsigned ub, us;
+    seq.divmod((unsigned)p, ub, us);
+    const int b = (int)ub, s = (int)us;
+
+    // (cos, sin) of the token's pairs: once per workgroup, by its first wave (as in qkv_rope_wave)
+    const int block_first = (int)blockIdx.y * WAVES * HEADS_PER_WAVE;
+    float c[VEC], sn[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; e++) { c[e] = 1.0f; sn[e] = 0.0f; }
+    if (block_first < head_num + kv_head_num) {  // workgroup-uniform
+        __shared__ float2 cs[HALF];
+        if (wave == 0 && lane < HALF) {
+            float2 coef = make_float2(1.0f, 0.0f);
+            if (lane < half_rot) coef = rope_coefficients(history_length[b] + s, tab.div[lane]);
+            cs[lane] = coef;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int e = 0; e < VEC; e++) {
+            const float2 t = cs[(g & 3) * VEC + e];   // pair index d = element index modulo 32
+            c[e] = t.x;
+            sn[e] = t.y;
         }
     }
-};
+    if (!live) return;
 
-static FastDiv make_fastdiv(unsigned d) {
-    FastDiv f;
-    f.d = d;
-    f.m = d <= 1 ? 0xffffffffu : (unsigned)(0x100000000ull / d);
-    return f;
+    float x[VEC];
+    Elem<__half>::unpack(raw, x);
+    if (bias) {
+        float bv[VEC];
+        Elem<__half>::unpack(braw, bv);
+#pragma unroll
+        for (int e = 0; e < VEC; e++) x[e] += bv[e];
+    }
+    __half* dst;
+    __half* cache = nullptr;
+    bool rotate = true;
+    if (h < head_num) {
+        dst = q + (((size_t)b * head_num + h) * seq_len + s) * HS;
+    } else {
+        const bool is_k = h < head_num + kv_head_num;
+        const int kvh = is_k ? h - head_num : h - head_num - kv_head_num;
+        __half* plane = is_k ? k : v;
+        dst = plane ? plane + (((size_t)b * kv_head_num + kvh) * seq_len + s) * HS : nullptr;
+        rotate = is_k;
+        const long long row = append_row(ap, history_length, b, s);
+        if (row >= 0)
+            cache = (is_k ? ap.k_cache : ap.v_cache) +
+                    (((size_t)b * kv_head_num + kvh) * (size_t)ap.max_seq_len + (size_t)row) * HS;
+    }
+    const bool upper = g >= 4;   // this lane holds x[d + 32]; its partner, 4 lanes down, holds x[d]
+    float y[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; e++) {
+        // partner = the lane 4 further on (lower half rows) or 4 further back (upper half rows).  A row
+        // rotation by n hands lane i the value of lane (i - n) mod 16: row_ror:12 serves lane banks 0
+        // and 2 of each row of 16 (they read lane i + 4), row_ror:4 banks 1 and 3 (lane i - 4)
+        unsigned other = __builtin_amdgcn_update_dpp(0u, __float_as_uint(x[e]), 0x12C, 0xf, 0x5, false);
+        other = __builtin_amdgcn_update_dpp(other, __float_as_uint(x[e]), 0x124, 0xf, 0xA, false);
+        const float xo = __uint_as_float(other);
+        const bool r = rotate && ((g & 3) * VEC + e) < half_rot;
+        // lower: c x[d] - s x[d + 32];  upper: c x[d + 32] + s x[d]   (rotate_pair, one half each)
+        const float rot = upper ? __fmaf_rn(c[e], x[e], sn[e] * xo) : __fmaf_rn(c[e], x[e], -(sn[e] * xo));
+        y[e] = r ? rot : x[e];
+    }
+    const vec16 out = Elem<__half>::pack(y);
+    if (dst) store16_sel<ST>(dst + col, out);
+    if (cache) store16_sel<ST>(cache + col, out);
 }
 
 // The common LLaMA shape (fp16, head size 128 fully rotated, q and kv head counts multiples of 32)
@@ -693,7 +800,7 @@ static int qkv_rope(void* q_, void* k_, void* v_, const void* qkv_, const void* 
         constexpr int HPB = (kWave / ((HS / 2) / Elem<T>::kVec)) * W;                              \
         dim3 g2((unsigned)token_num, (unsigned)((head_num + 2 * kv_head_num + HPB - 1) / HPB));    \
         hipLaunchKernelGGL((qkv_rope_wave<T, HS, K, W>), g2, dim3(kWave * W), 0, s, q, k, v, qkv,   \
-                           bias, padding_offset, history_length, batch, seq_len, head_num,         \
+                           bias, padding_offset, history_length, positions, fd, head_num,          \
                            kv_head_num, half_rot, tab, ap);                                        \
     } while (0)
 #define ISP_QKV_LAUNCH_K(HS, W)                                                                    \
@@ -709,6 +816,10 @@ static int qkv_rope(void* q_, void* k_, void* v_, const void* qkv_, const void* 
         else ISP_QKV_LAUNCH_K(HS, 4);                                                              \
     } while (0)
     const int head_groups_max = 65535 * 4;  // grid.y limit, 4 heads per workgroup at least
+    // the vector kernels keep padded positions in 32 bits and divide by seq_len with a multiply-high
+    const bool positions_ok = (unsigned long long)batch * (unsigned long long)seq_len <= 0x7fffffffull;
+    const unsigned positions = positions_ok ? (unsigned)batch * (unsigned)seq_len : 0u;
+    const FastDiv fd = make_fastdiv((unsigned)seq_len);
     // lean kernel: fp16, 128-element heads fully rotated, whole groups of 32 q / k / v heads, offsets
     // inside a group and positions inside the batch in 32 bits; ISP_TUNE_QKV_WAVES = 1, 2, 4 opts out
     const int waves_knob = tuning(ISP_TUNE_QKV_WAVES);
@@ -717,12 +828,9 @@ static int qkv_rope(void* q_, void* k_, void* v_, const void* qkv_, const void* 
                          (head_num + 2 * kv_head_num) / 32 <= 65535 &&
                          (unsigned long long)seq_len * 256ull * 32ull <= 0xffffffffull &&
                          (unsigned long long)max_seq_len * 256ull * 32ull <= 0xffffffffull &&
-                         (unsigned long long)batch * (unsigned long long)seq_len <= 0x7fffffffull &&
-                         (waves_knob <= 0 || waves_knob >= 8);
+                         positions_ok && (waves_knob <= 0 || waves_knob >= 8);
     if (lean_ok) {
         const dim3 g2((unsigned)token_num, (unsigned)((head_num + 2 * kv_head_num) / 32));
-        const unsigned positions = (unsigned)batch * (unsigned)seq_len;
-        const FastDiv fd = make_fastdiv((unsigned)seq_len);
         __half* qh = reinterpret_cast<__half*>(q);
         __half* kh = reinterpret_cast<__half*>(k);
         __half* vh = reinterpret_cast<__half*>(v);
@@ -748,10 +856,28 @@ static int qkv_rope(void* q_, void* k_, void* v_, const void* qkv_, const void* 
 #undef ISP_QKV_LEAN_2
 #undef ISP_QKV_LEAN
         e = hipGetLastError();
-    } else if (vec_ok && head_size == 128 && head_num + 2 * kv_head_num <= head_groups_max) {
+    } else if (vec_ok && positions_ok && head_size == 128 && head_num + 2 * kv_head_num <= head_groups_max) {
         ISP_QKV_LAUNCH_WAVE(128);
         e = hipGetLastError();
-    } else if (vec_ok && head_size == 64 && head_num + 2 * kv_head_num <= head_groups_max) {
+    } else if (sizeof(T) == 2 && vec_ok && positions_ok && head_size == 64 && waves_knob <= 0 &&
+               head_num + 2 * kv_head_num <= head_groups_max) {
+        // fp16 rows of 128 bytes: one vector per lane, 8 lanes per row, 4 waves = 32 heads per workgroup
+        constexpr int W = 4;
+        const dim3 g2((unsigned)token_num, (unsigned)((head_num + 2 * kv_head_num + 8 * W - 1) / (8 * W)));
+        KvAppend<__half> aph = {reinterpret_cast<__half*>(ap.k_cache), reinterpret_cast<__half*>(ap.v_cache),
+                                ap.input_length, ap.max_seq_len};
+#define ISP_QKV_ROWS64(K)                                                                          \
+    hipLaunchKernelGGL((qkv_rope_rows64_f16<K, W>), g2, dim3(kWave * W), 0, s,                      \
+                       reinterpret_cast<__half*>(q), reinterpret_cast<__half*>(k),                 \
+                       reinterpret_cast<__half*>(v), reinterpret_cast<const __half*>(qkv),         \
+                       reinterpret_cast<const __half*>(bias), padding_offset, history_length,      \
+                       positions, fd, head_num, kv_head_num, half_rot, tab, aph)
+        if (kind == kStoreThrough) ISP_QKV_ROWS64(kStoreThrough);
+        else if (kind == kStoreStream) ISP_QKV_ROWS64(kStoreStream);
+        else ISP_QKV_ROWS64(kStorePlain);
+#undef ISP_QKV_ROWS64
+        e = hipGetLastError();
+    } else if (vec_ok && positions_ok && head_size == 64 && head_num + 2 * kv_head_num <= head_groups_max) {
         ISP_QKV_LAUNCH_WAVE(64);
         e = hipGetLastError();
     } else {
