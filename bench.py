@@ -482,6 +482,25 @@ def context_layer_record(torch, steps, warmup, stream):
             "note": "library kernels via the C ABI; GEMMs and attention are torch library calls"}
 
 
+def context_layer_cpp_record(torch, steps, warmup):
+    """The same layer through the C++ layer class (launch* kernels + hipBLASLt GEMMs called directly, padded
+    batched attention): runs build/bin/bench_context_layer in a child process and returns its JSON record."""
+    import subprocess
+    exe = os.path.join(ROOT, "build", "bin", "bench_context_layer")
+    if not os.path.exists(exe):
+        return {"error": "build/bin/bench_context_layer is missing (python -m inferspore_amd.build)"}
+    lens = [str(int(v)) for v in bench_lengths(torch).tolist()]
+    try:
+        p = subprocess.run([exe, str(max(10, steps // 10)), str(max(3, warmup // 4)), "512"] + lens,
+                           stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=300)
+        lines = [l for l in p.stdout.splitlines() if l.startswith("{")]
+        if p.returncode != 0 or not lines:
+            return {"error": p.stdout[-400:]}
+        return json.loads(lines[-1])
+    except (OSError, subprocess.SubprocessError, ValueError) as e:
+        return {"error": str(e)}
+
+
 def decode_sequence_record(torch, stream):
     """The launch-bound side: one decode step's worth of this library's kernels (batch 16: fused norm,
     decode RoPE, KV append, KV broadcast, SwiGLU, RMSNorm) issued eagerly and replayed from a captured
@@ -816,6 +835,7 @@ def main():
         layer["library_kernels_ms_estimate"] = est
         layer["library_kernels_share"] = est / layer["ms_per_layer"]
         config["context_layer"] = layer
+        config["context_layer_cpp"] = context_layer_cpp_record(torch, a.steps, a.warmup)
         config["decode_sequence"] = decode_sequence_record(torch, stream)
     if not a.kernels_only:
         # cache-resident rates (one buffer set, no rotation): the hot-path configurations by default, every

@@ -16,6 +16,22 @@ void launchAddFusedQKVBiasTransposeAndRoPE(TensorWrapper<T>* q_buf, TensorWrappe
                                            TensorWrapper<int>* input_length,
                                            LLaMAAttentionStaticParams& params);
 
+// The same step with launchConcatKVCache fused in (no counterpart in the reference, which runs the two
+// launchers one after the other, src/kernels/concat_past_kv.cu:76-113): the k and v rows go straight
+// to k_cache / v_cache [layers, batch, kv_head_num, max_seq_len, head_size] at layer layer_id (a host
+// tensor, as in launchConcatKVCache) and row history_length[b] + s; no padded k / v buffers are
+// written.  kv_head_num and max_seq_len are taken from the cache's shape.
+template <typename T>
+void launchAddFusedQKVBiasTransposeRoPEAndConcatKV(TensorWrapper<T>* q_buf, TensorWrapper<T>* QKV,
+                                                   BaseWeight<T>& qkv,
+                                                   TensorWrapper<int>* padding_offset,
+                                                   TensorWrapper<int>* history_length,
+                                                   TensorWrapper<int>* input_length,
+                                                   TensorWrapper<int>* layer_id,
+                                                   TensorWrapper<T>* k_cache,
+                                                   TensorWrapper<T>* v_cache,
+                                                   LLaMAAttentionStaticParams& params);
+
 // launchRoPE -- same declaration as the reference's src/kernels/qkv_bias_and_RoPE.h:22-25 (decode
 // phase): in-place rotate-half RoPE on qkv_buf [1, 96, 128] at timestep step - 1; `step` is a host
 // (CPU) tensor.  The reference's checks (batch 1, 96 heads of 128, 32 q heads) are kept.

@@ -1,0 +1,85 @@
+// One LLaMA context-decoder (prefill) layer in C++ over the reference's data model: TensorWrapper /
+// TensorMap activations, LlamaLayerWeight weights, a BaseAllocator for the intermediate buffers.
+//
+// The reference ships the kernels and the weight containers but not the layer code that joins them
+// (no src/layers in its tree; its factory constructs an absent Llama<T>, src/utils/model_utils.h:40).
+// This class is that join for one layer, in the order the kernels' comments and the weight layout
+// imply (src/kernels/linear.cu:7-15, src/weights/llama/layer_weights.cc:19-41,
+// src/kernels/fused_addresidual_norm.cu:30,61):
+//
+//   qkv      = decoder_input x Wqkv^T                      GEMM   [tokens, H] -> [tokens, heads, hs]
+//   q, cache = launchAddFusedQKVBiasTransposeRoPEAndConcatKV    bias + RoPE + re-pad + KV append
+//   k, v     = launchRepeatKVCache                          cache -> [batch, head_num, max_k_len, hs]
+//   scores   = q x k^T (batched GEMM) ; masked, scaled softmax ; ctx = p x v (batched GEMM)
+//   packed   = launchTransposeOutRemovePadding              [batch, heads, max_q, hs] -> [tokens, H]
+//   attn     = packed x Wo^T                                GEMM
+//   launchFusedAddBiasResidualRMSNorm(residual, attn, o-bias, ffn_norm)     residual += attn ; attn := norm
+//   gate_up  = attn x Wgate_up^T                            GEMM   -> [tokens, 2, inter]
+//   act      = launchAct(gate_up)                           SwiGLU
+//   out      = act x Wdown^T                                GEMM
+//   launchFusedAddBiasResidualRMSNorm(residual, out, down-bias, next layer's attn_norm)
+//
+// Every memory-bound step is one of this library's launch* entry points; the five dense GEMMs and the
+// two batched attention GEMMs are hipBLASLt calls made here; the softmax between them is a plain
+// kernel of this file's own (attention is not one of the optimised kernels of this library).
+// Everything runs on the null stream, as the reference's launchers do.
+//
+// forward() tensors (names as the kernels' parameters):
+//   inputs   "decoder_input"    T   [num_tokens, hidden]   normalised by this layer's attn_norm; used as scratch
+//            "decoder_residual" T   [num_tokens, hidden]   updated in place
+//            "padding_offset"   int [batch, max_q_len]     from launchCalPaddingoffset
+//            "history_length", "input_length", "context_length"   int [batch]   (device)
+//            "layer_id"         int [1]                    host tensor
+//   outputs  "decoder_output"   T   [num_tokens, hidden]   the next layer's normalised input
+//            "all_k_cache", "all_v_cache"   T [layers, batch, kv_head_num, max_seq_len, head_size]
+#pragma once
+#include <memory>
+
+#include "src/memory/allocator/base_allocator.h"
+#include "src/models/llama/llama_params.h"
+#include "src/utils/tensor.h"
+#include "src/weights/llama/layer_weights.h"
+
+namespace isp_layers {
+class GemmEngine;  // hipBLASLt handle, workspace and per-shape algorithm cache
+}
+
+template <typename T>
+class LlamaContextDecoderLayer {
+public:
+    LlamaContextDecoderLayer(int head_num, int kv_head_num, int head_size, int inter_size,
+                             const LLaMAAttentionStaticParams& attn_params, float rmsnorm_eps,
+                             BaseAllocator* allocator);
+    ~LlamaContextDecoderLayer();
+    LlamaContextDecoderLayer(const LlamaContextDecoderLayer&) = delete;
+    LlamaContextDecoderLayer& operator=(const LlamaContextDecoderLayer&) = delete;
+
+    // (Re)allocates the intermediate buffers for these extents; forward() calls it when they grow.
+    void allocForForward(const LLaMAAttentionDynParams& dyn);
+    void freeBuf();
+
+    // next_attn_norm: gamma [hidden] of the following layer's attention norm (or the model's final norm).
+    void forward(TensorMap& inputs, LlamaLayerWeight<T>& weights, LayerNormWeight<T>& next_attn_norm,
+                 TensorMap& outputs, const LLaMAAttentionDynParams& dyn);
+
+    // Device bytes the intermediate buffers of one call with these extents take.
+    size_t workspaceBytes(const LLaMAAttentionDynParams& dyn) const;
+
+private:
+    int head_num_, kv_head_num_, head_size_, inter_size_, hidden_;
+    LLaMAAttentionStaticParams attn_params_;
+    float eps_;
+    BaseAllocator* allocator_;
+    std::unique_ptr<isp_layers::GemmEngine> gemm_;
+
+    LLaMAAttentionDynParams allocated_;
+    T* qkv_buf_ = nullptr;      // [tokens, head_num + 2 kv_head_num, head_size]
+    T* q_buf_ = nullptr;        // [batch, head_num, max_q_len, head_size]
+    T* k_all_ = nullptr;        // [batch, head_num, max_k_len, head_size]
+    T* v_all_ = nullptr;
+    T* scores_ = nullptr;       // [batch, head_num, max_q_len, max_k_len]
+    T* ctx_ = nullptr;          // [batch, head_num, max_q_len, head_size]
+    T* ctx_packed_ = nullptr;   // [tokens, head_num, head_size]
+    T* gate_up_ = nullptr;      // [tokens, 2, inter]
+    T* act_ = nullptr;          // [tokens, inter]
+};

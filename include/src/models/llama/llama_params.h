@@ -9,3 +9,15 @@ struct LLaMAAttentionStaticParams {
     int max_position_embeddings = 2048;
     bool use_dynamic_ntk = false;  // placeholder in the reference as well
 };
+
+// Per-call extents of the attention / decoder layers.  The reference's kernels take them from tensor
+// shapes; the layer code (which the reference does not ship) needs them before the tensors exist,
+// to size its buffers.
+struct LLaMAAttentionDynParams {
+    int batch_size = 0;
+    int num_tokens = 0;   // valid (un-padded) tokens of the batch
+    int max_q_len = 0;    // longest query of the batch: the padded sequence extent of q
+    int max_k_len = 0;    // longest context (history + query) of the batch
+    int num_layers = 0;
+    bool is_ctx = true;
+};

@@ -6,6 +6,7 @@
 Outputs (git-ignored, but they travel with the source tree to a GPU machine):
     inferspore_amd/lib/libinferspore_amd.so     HIP kernels + the C ABI (include/inferspore_amd.h)
     inferspore_amd/lib/libinferspore_launch.so  the C++ `launch*` shims over the C ABI
+    inferspore_amd/lib/libinferspore_layers.so  the C++ context-decoder layer (launch* + hipBLASLt GEMMs)
     build/bin/test_*                            reference-style C++ call-site programs
 """
 import argparse
@@ -33,6 +34,8 @@ HIPCC_FLAGS = [
 
 LIB_KERNELS = os.path.join(LIBDIR, "libinferspore_amd.so")
 LIB_LAUNCH = os.path.join(LIBDIR, "libinferspore_launch.so")
+LIB_LAYERS = os.path.join(LIBDIR, "libinferspore_layers.so")
+LAYERS = os.path.join(CSRC, "layers")
 
 
 def _run(cmd):
@@ -73,6 +76,18 @@ def build(verbose=False, jobs=8, cpp_tests=True):
     if os.path.exists(launch_src):
         _run([hipcc()] + HIPCC_FLAGS + ["-x", "hip", "-shared", launch_src, "-o", LIB_LAUNCH,
                                         "-L" + LIBDIR, "-linferspore_amd", "-Wl,-rpath,$ORIGIN"])
+        if os.path.isdir(LAYERS):
+            names = sorted(f for f in os.listdir(LAYERS) if f.endswith((".hip", ".cc")))
+            layer_srcs = [os.path.join(LAYERS, f) for f in names if not f.endswith("_main.cc")]
+            _run([hipcc()] + HIPCC_FLAGS + ["-x", "hip", "-shared"] + layer_srcs + [
+                "-o", LIB_LAYERS, "-L" + LIBDIR, "-linferspore_launch", "-linferspore_amd",
+                "-L/opt/rocm/lib", "-lhipblaslt", "-Wl,-rpath,$ORIGIN", "-Wl,-rpath,/opt/rocm/lib"])
+            for f in names:   # stand-alone programs over the layers library: <name>_main.cc -> build/bin/<name>
+                if f.endswith("_main.cc"):
+                    _run([hipcc()] + HIPCC_FLAGS + ["-x", "hip", os.path.join(LAYERS, f), "-o",
+                                                    os.path.join(BINDIR, f[:-len("_main.cc")]),
+                                                    "-L" + LIBDIR, "-linferspore_layers", "-linferspore_launch",
+                                                    "-linferspore_amd", "-Wl,-rpath,$ORIGIN/../../inferspore_amd/lib"])
         if cpp_tests and os.path.isdir(CPPTESTS):
             # the test programs (not the libraries) link the CPU oracle they check against
             oracle_dir = os.path.join(ROOT, "oracle")
@@ -84,7 +99,7 @@ def build(verbose=False, jobs=8, cpp_tests=True):
                 exe = os.path.join(BINDIR, os.path.splitext(f)[0])
                 return _run([hipcc()] + HIPCC_FLAGS + [
                     "-x", "hip", os.path.join(CPPTESTS, f), "-o", exe, "-I" + oracle_dir,
-                    "-L" + LIBDIR, "-linferspore_launch", "-linferspore_amd",
+                    "-L" + LIBDIR, "-linferspore_layers", "-linferspore_launch", "-linferspore_amd",
                     "-L" + oracle_dir, "-lisp_oracle",
                     # relative to build/bin, so the tree can be moved or mounted elsewhere
                     "-Wl,-rpath,$ORIGIN/../../inferspore_amd/lib", "-Wl,-rpath,$ORIGIN/../../oracle"])
@@ -95,7 +110,7 @@ def build(verbose=False, jobs=8, cpp_tests=True):
 
 
 def clean():
-    for p in (LIB_KERNELS, LIB_LAUNCH):
+    for p in (LIB_KERNELS, LIB_LAUNCH, LIB_LAYERS):
         if os.path.exists(p):
             os.remove(p)
     shutil.rmtree(os.path.join(ROOT, "build"), ignore_errors=True)

@@ -8,8 +8,8 @@ order a model runs them:
 
     normed, residual                       (packed [tokens, H]; `normed` = RMSNorm(residual) by attn_norm)
     qkv      = normed @ Wqkv                                 library GEMM (out of this library's scope)
-    q, k, v  = add_fused_qkv_bias_transpose_and_rope(qkv)    * this library
-    cache   += k, v ; k_all, v_all = repeat(cache)           * this library
+    q, cache += k, v = add_fused_qkv_bias_transpose_rope_and_append(qkv)    * this library
+    k_all, v_all = repeat(cache)                             * this library
     ctx      = softmax(q k^T / sqrt(d) + mask) v             library attention (out of scope)
     packed   = transpose_out_remove_padding(ctx)             * this library
     attn_out = packed @ Wo                                   library GEMM
@@ -66,8 +66,6 @@ class BatchState:
         hidden = head_num * head_size
         z = lambda *s: torch.zeros(s, dtype=dtype, device=dev)
         self.q = z(self.batch, head_num, max_q_len, head_size)
-        self.k = z(self.batch, kv_head_num, max_q_len, head_size)
-        self.v = z(self.batch, kv_head_num, max_q_len, head_size)
         self.k_cache = z(layers, self.batch, kv_head_num, max_seq_len, head_size)
         self.v_cache = z(layers, self.batch, kv_head_num, max_seq_len, head_size)
         self.k_all = z(self.batch, head_num, self.max_k_len, head_size)
@@ -94,9 +92,10 @@ def context_decoder_layer(normed, residual, w, state, layer_id, next_norm_gamma,
     st = state
     qkv = normed @ w.qkv                                                       # [tokens, 3H]
     qkv = qkv.view(st.tokens, st.head_num + 2 * st.kv_head_num, st.head_size)
-    ops.add_fused_qkv_bias_transpose_and_rope(st.q, st.k, st.v, qkv, w.qkv_bias, st.padding_offset, st.history,
-                                              st.lengths, rotary_dim, rotary_base)
-    ops.concat_kv_cache(st.k, st.v, layer_id, st.lengths, st.history, st.k_cache, st.v_cache)
+    # bias + RoPE + re-pad of q, with k and v written straight into the cache (one launch, no padded k / v)
+    ops.add_fused_qkv_bias_transpose_rope_and_append(st.q, None, None, st.k_cache, st.v_cache, layer_id, qkv,
+                                                     w.qkv_bias, st.padding_offset, st.history, st.lengths,
+                                                     rotary_dim, rotary_base)
     ops.repeat_kv_cache(st.k_cache, st.v_cache, st.context, layer_id, st.k_all, st.v_all)
     ctx = torch.nn.functional.scaled_dot_product_attention(st.q, st.k_all, st.v_all, attn_mask=st.mask,
                                                            scale=1.0 / math.sqrt(st.head_size))

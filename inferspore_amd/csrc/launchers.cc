@@ -24,6 +24,7 @@ struct Abi<float> {
     static constexpr auto rmsnorm = isp_rmsnorm_f32;
     static constexpr auto fused_norm = isp_fused_add_bias_residual_rmsnorm_f32;
     static constexpr auto qkv = isp_qkv_bias_rope_transpose_f32;
+    static constexpr auto qkv_append = isp_qkv_bias_rope_transpose_append_f32;
     static constexpr auto swiglu = isp_swiglu_f32;
     static constexpr auto rope_decode = isp_rope_decode_f32;
     static constexpr auto transpose_remove_padding = isp_transpose_remove_padding_f32;
@@ -36,6 +37,7 @@ struct Abi<half> {
     static constexpr auto rmsnorm = isp_rmsnorm_f16;
     static constexpr auto fused_norm = isp_fused_add_bias_residual_rmsnorm_f16;
     static constexpr auto qkv = isp_qkv_bias_rope_transpose_f16;
+    static constexpr auto qkv_append = isp_qkv_bias_rope_transpose_append_f16;
     static constexpr auto swiglu = isp_swiglu_f16;
     static constexpr auto rope_decode = isp_rope_decode_f16;
     static constexpr auto transpose_remove_padding = isp_transpose_remove_padding_f16;
@@ -118,6 +120,39 @@ void launchAddFusedQKVBiasTransposeAndRoPE(TensorWrapper<T>* q_buf, TensorWrappe
                           params.rotary_embedding_dim, params.rotary_embedding_base,
                           params.max_position_embeddings, params.use_dynamic_ntk ? 1 : 0, nullptr),
               "launchAddFusedQKVBiasTransposeAndRoPE");
+}
+
+// shapes as above; kv_head_num and max_seq_len from the cache [layers, batch, kv_head_num, max_seq_len, hs]
+template <typename T>
+void launchAddFusedQKVBiasTransposeRoPEAndConcatKV(TensorWrapper<T>* q_buf, TensorWrapper<T>* QKV,
+                                                   BaseWeight<T>& qkv,
+                                                   TensorWrapper<int>* padding_offset,
+                                                   TensorWrapper<int>* history_length,
+                                                   TensorWrapper<int>* input_length,
+                                                   TensorWrapper<int>* layer_id,
+                                                   TensorWrapper<T>* k_cache,
+                                                   TensorWrapper<T>* v_cache,
+                                                   LLaMAAttentionStaticParams& params) {
+    const int token_num = QKV->shape[0];
+    const int qkv_head_num = QKV->shape[1];
+    const int head_size = QKV->shape[2];
+    const int batch_size = q_buf->shape[0];
+    const int head_num = q_buf->shape[1];
+    const int seq_len = q_buf->shape[2];
+    const int kv_head_num = (qkv_head_num - head_num) / 2;
+    LLM_CHECK_WITH_INFO(k_cache->shape.size() == 5 && k_cache->shape == v_cache->shape,
+                        "k / v cache should be [layers, batch, kv heads, max seq len, head size]");
+    LLM_CHECK_WITH_INFO(k_cache->shape[1] == batch_size && k_cache->shape[2] == kv_head_num &&
+                            k_cache->shape[4] == head_size,
+                        "k / v cache extents should match the qkv buffer's");
+    const int layer = layer_id->getVal();
+    LLM_CHECK_WITH_INFO(layer >= 0 && layer < k_cache->shape[0], "layer id outside the cache");
+    expect_ok(Abi<T>::qkv_append(q_buf->data, nullptr, nullptr, k_cache->data, v_cache->data, layer,
+                                 k_cache->shape[3], QKV->data, qkv.bias, padding_offset->data,
+                                 history_length->data, input_length->data, batch_size, seq_len,
+                                 token_num, head_num, kv_head_num, head_size,
+                                 params.rotary_embedding_dim, params.rotary_embedding_base, nullptr),
+              "launchAddFusedQKVBiasTransposeRoPEAndConcatKV");
 }
 
 // reference: src/kernels/act_kernel.cu:57-71 (the shape[1] == 2 check at :61)
@@ -206,6 +241,10 @@ void launchRepeatKVCache(TensorWrapper<T>* k_cache_src, TensorWrapper<T>* v_cach
     template void launchAddFusedQKVBiasTransposeAndRoPE(                                            \
         TensorWrapper<T>*, TensorWrapper<T>*, TensorWrapper<T>*, TensorWrapper<T>*, BaseWeight<T>&, \
         TensorWrapper<int>*, TensorWrapper<int>*, TensorWrapper<int>*, LLaMAAttentionStaticParams&); \
+    template void launchAddFusedQKVBiasTransposeRoPEAndConcatKV(                                    \
+        TensorWrapper<T>*, TensorWrapper<T>*, BaseWeight<T>&, TensorWrapper<int>*,                  \
+        TensorWrapper<int>*, TensorWrapper<int>*, TensorWrapper<int>*, TensorWrapper<T>*,           \
+        TensorWrapper<T>*, LLaMAAttentionStaticParams&);                                            \
     template void launchAct(TensorWrapper<T>*, TensorWrapper<T>*);                                  \
     template void launchRoPE(TensorWrapper<T>*, TensorWrapper<int>*, LLaMAAttentionStaticParams&);  \
     template void launchTransposeOutRemovePadding(TensorWrapper<T>*, TensorWrapper<int>*,           \

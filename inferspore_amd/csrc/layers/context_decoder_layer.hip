@@ -1,0 +1,370 @@
+// LlamaContextDecoderLayer: one LLaMA prefill layer over the reference's data model (see the header
+// for the sequence).  This file holds the parts that are not this library's launch* kernels: the
+// hipBLASLt GEMM calls (shape cases of the reference's src/kernels/linear.cu:7-15, 67-109) and a plain
+// masked softmax for the attention scores.
+#include "src/layers/decoder/context_decoder_layer.h"
+
+#include <hipblaslt/hipblaslt.h>
+
+#include <cmath>
+#include <map>
+#include <string>
+#include <tuple>
+
+#include "src/kernels/act_kernel.h"
+#include "src/kernels/fused_addresidual_norm.h"
+#include "src/kernels/fused_transpose_and_remv_pad.h"
+#include "src/kernels/qkv_bias_and_RoPE.h"
+#include "src/kernels/repeat_kv.h"
+#include "src/utils/macro.h"
+
+namespace isp_layers {
+
+#define ISP_LT_CHECK(call)                                                                          \
+    do {                                                                                            \
+        const hipblasStatus_t isp_lt_status_ = (call);                                              \
+        LLM_CHECK_WITH_INFO(isp_lt_status_ == HIPBLAS_STATUS_SUCCESS,                               \
+                            std::string("hipBLASLt call failed with status ") +                     \
+                                std::to_string((int)isp_lt_status_) + ": " #call);                  \
+    } while (0)
+
+template <typename T>
+struct LtType;
+template <>
+struct LtType<float> {
+    static constexpr hipDataType value = HIP_R_32F;
+};
+template <>
+struct LtType<half> {
+    static constexpr hipDataType value = HIP_R_16F;
+};
+
+// Row-major C[m, n] = alpha * A[m, k] x op(W), fp32 accumulation, optionally strided-batched.
+//   w_is_nk:  W is stored [n, k] (a weight kept [out_features, in_features], or the keys of
+//             q x k^T), else [k, n].
+// hipBLASLt is column-major, so the call computes C^T = op(W)^T x A^T: its "A" operand is W, its
+// "B" operand is the activation, and a row-major [r, c] matrix is a column-major [c, r] one.
+class GemmEngine {
+public:
+    explicit GemmEngine(BaseAllocator* allocator) : allocator_(allocator) {
+        ISP_LT_CHECK(hipblasLtCreate(&handle_));
+        workspace_ = allocator_->UnifyMalloc(nullptr, kWorkspaceBytes, false);
+        ISP_LT_CHECK(hipblasLtMatmulPreferenceCreate(&pref_));
+        const uint64_t ws = kWorkspaceBytes;
+        ISP_LT_CHECK(hipblasLtMatmulPreferenceSetAttribute(pref_, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &ws,
+                                                           sizeof(ws)));
+    }
+    ~GemmEngine() {
+        for (auto& kv : plans_) destroy(kv.second);
+        if (pref_) (void)hipblasLtMatmulPreferenceDestroy(pref_);
+        if (workspace_) allocator_->UnifyFree(workspace_, false);
+        if (handle_) (void)hipblasLtDestroy(handle_);
+    }
+    GemmEngine(const GemmEngine&) = delete;
+    GemmEngine& operator=(const GemmEngine&) = delete;
+
+    void matmul(hipDataType type, const void* a, const void* w, void* c, int m, int n, int k, bool w_is_nk,
+                int lda, int ldw, int ldc, int batch = 1, long long stride_a = 0, long long stride_w = 0,
+                long long stride_c = 0, float alpha = 1.0f) {
+        if (m == 0 || n == 0 || batch == 0) return;
+        const Key key{(int)type, m, n, k, w_is_nk ? 1 : 0, lda, ldw, ldc, batch, stride_a, stride_w, stride_c};
+        auto it = plans_.find(key);
+        if (it == plans_.end()) it = plans_.emplace(key, plan(type, key)).first;
+        const Plan& p = it->second;
+        const float beta = 0.0f;
+        ISP_LT_CHECK(hipblasLtMatmul(handle_, p.desc, &alpha, w, p.w, a, p.a, &beta, c, p.c, c, p.c, &p.algo,
+                                     workspace_, kWorkspaceBytes, nullptr));
+    }
+
+private:
+    static constexpr size_t kWorkspaceBytes = 32u << 20;
+    using Key = std::tuple<int, int, int, int, int, int, int, int, int, long long, long long, long long>;
+    struct Plan {
+        hipblasLtMatmulDesc_t desc = nullptr;
+        hipblasLtMatrixLayout_t w = nullptr, a = nullptr, c = nullptr;
+        hipblasLtMatmulAlgo_t algo;
+    };
+
+    static void batched(hipblasLtMatrixLayout_t layout, int batch, long long stride) {
+        if (batch <= 1) return;
+        const int32_t count = batch;
+        const int64_t offset = stride;
+        ISP_LT_CHECK(hipblasLtMatrixLayoutSetAttribute(layout, HIPBLASLT_MATRIX_LAYOUT_BATCH_COUNT, &count, sizeof(count)));
+        ISP_LT_CHECK(hipblasLtMatrixLayoutSetAttribute(layout, HIPBLASLT_MATRIX_LAYOUT_STRIDED_BATCH_OFFSET, &offset,
+                                                       sizeof(offset)));
+    }
+
+    Plan plan(hipDataType type, const Key& key) {
+        int m, n, k, nk, lda, ldw, ldc, batch, t;
+        long long sa, sw, sc;
+        std::tie(t, m, n, k, nk, lda, ldw, ldc, batch, sa, sw, sc) = key;
+        Plan p;
+        ISP_LT_CHECK(hipblasLtMatmulDescCreate(&p.desc, HIPBLAS_COMPUTE_32F, HIP_R_32F));
+        const hipblasOperation_t op_w = nk ? HIPBLAS_OP_T : HIPBLAS_OP_N, op_a = HIPBLAS_OP_N;
+        ISP_LT_CHECK(hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_TRANSA, &op_w, sizeof(op_w)));
+        ISP_LT_CHECK(hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_TRANSB, &op_a, sizeof(op_a)));
+        // column-major views: W [n, k] row-major = [k, n] column-major (transposed by op_w);
+        // W [k, n] row-major = [n, k] column-major; A [m, k] row-major = [k, m]; C [m, n] = [n, m]
+        if (nk) ISP_LT_CHECK(hipblasLtMatrixLayoutCreate(&p.w, type, (uint64_t)k, (uint64_t)n, ldw));
+        else ISP_LT_CHECK(hipblasLtMatrixLayoutCreate(&p.w, type, (uint64_t)n, (uint64_t)k, ldw));
+        ISP_LT_CHECK(hipblasLtMatrixLayoutCreate(&p.a, type, (uint64_t)k, (uint64_t)m, lda));
+        ISP_LT_CHECK(hipblasLtMatrixLayoutCreate(&p.c, type, (uint64_t)n, (uint64_t)m, ldc));
+        batched(p.w, batch, sw);
+        batched(p.a, batch, sa);
+        batched(p.c, batch, sc);
+        hipblasLtMatmulHeuristicResult_t found[1];
+        int count = 0;
+        ISP_LT_CHECK(hipblasLtMatmulAlgoGetHeuristic(handle_, p.desc, p.w, p.a, p.c, p.c, pref_, 1, found, &count));
+        LLM_CHECK_WITH_INFO(count > 0, "hipBLASLt offers no algorithm for a GEMM of this layer");
+        p.algo = found[0].algo;
+        return p;
+    }
+
+    static void destroy(Plan& p) {
+        if (p.w) (void)hipblasLtMatrixLayoutDestroy(p.w);
+        if (p.a) (void)hipblasLtMatrixLayoutDestroy(p.a);
+        if (p.c) (void)hipblasLtMatrixLayoutDestroy(p.c);
+        if (p.desc) (void)hipblasLtMatmulDescDestroy(p.desc);
+    }
+
+    BaseAllocator* allocator_;
+    hipblasLtHandle_t handle_ = nullptr;
+    hipblasLtMatmulPreference_t pref_ = nullptr;
+    void* workspace_ = nullptr;
+    std::map<Key, Plan> plans_;
+};
+
+__device__ __forceinline__ float to_float(float x) { return x; }
+__device__ __forceinline__ float to_float(half x) { return __half2float(x); }
+__device__ __forceinline__ void from_float(float x, float* p) { *p = x; }
+__device__ __forceinline__ void from_float(float x, half* p) { *p = __float2half_rn(x); }
+
+__device__ __forceinline__ float block_reduce(float v, bool take_max, float* shared) {
+    for (int off = 32; off > 0; off >>= 1) {
+        const float o = __shfl_xor(v, off, 64);
+        v = take_max ? fmaxf(v, o) : v + o;
+    }
+    const int wave = threadIdx.x / 64, waves = blockDim.x / 64;
+    __syncthreads();  // `shared` may still be read from the previous reduction
+    if ((threadIdx.x % 64) == 0) shared[wave] = v;
+    __syncthreads();
+    v = shared[0];
+    for (int w = 1; w < waves; w++) v = take_max ? fmaxf(v, shared[w]) : v + shared[w];
+    return v;
+}
+
+// In place on scores [batch, head_num, max_q_len, max_k_len]: row (b, h, q) becomes
+// softmax(scale * scores) over the keys query q may see -- key positions <= history_length[b] + q and
+// < context_length[b] -- and zero elsewhere; rows of padded queries (q >= input_length[b]) become zero.
+// What the reference does with launchBuildCausalMasks + launchScaleMaskAndSoftmax
+// (src/kernels/build_casual_mask.cu:5-42, attn_softmax_kernel.cu:50-125), with the mask computed
+// from the lengths instead of read from a [batch, q, k] tensor.  fp32 arithmetic.
+template <typename T>
+__global__ __launch_bounds__(256) void masked_scaled_softmax(T* scores, const int* history_length,
+                                                             const int* input_length,
+                                                             const int* context_length, int head_num,
+                                                             int max_q_len, int max_k_len, float scale) {
+    __shared__ float shared[4];
+    const int q = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+    T* row = scores + (((size_t)b * head_num + h) * max_q_len + q) * (size_t)max_k_len;
+    int visible = 0;
+    if (q < input_length[b]) {
+        visible = history_length[b] + q + 1;
+        if (visible > context_length[b]) visible = context_length[b];
+        if (visible > max_k_len) visible = max_k_len;
+    }
+    float m = -INFINITY;
+    for (int i = threadIdx.x; i < visible; i += blockDim.x) m = fmaxf(m, scale * to_float(row[i]));
+    m = block_reduce(m, true, shared);
+    float sum = 0.0f;
+    for (int i = threadIdx.x; i < visible; i += blockDim.x) sum += expf(scale * to_float(row[i]) - m);
+    sum = block_reduce(sum, false, shared);
+    const float inv = visible > 0 ? 1.0f / sum : 0.0f;
+    for (int i = threadIdx.x; i < max_k_len; i += blockDim.x) {
+        const float p = i < visible ? expf(scale * to_float(row[i]) - m) * inv : 0.0f;
+        from_float(p, row + i);
+    }
+}
+
+}  // namespace isp_layers
+
+namespace {
+
+template <typename T>
+TensorWrapper<T>* as(Tensor* t, const char* name) {
+    LLM_CHECK_WITH_INFO(t->dtype == getTensorType<T>(), std::string(name) + " has the wrong element type");
+    return static_cast<TensorWrapper<T>*>(t);
+}
+
+// Whether a weight declared [rows, cols] is stored [out_features, in_features] (the reference's
+// constructor, layer_weights.cc:23,26,36,38) or [in_features, out_features] (the non-transposed case
+// of its GEMM wrapper, linear.cu:36-39).  A square weight is taken to be [out, in].
+template <typename T>
+bool stored_out_in(const BaseWeight<T>& w, int out_features, int in_features, const char* name) {
+    LLM_CHECK_WITH_INFO(w.data != nullptr && w.shape.size() == 2, std::string(name) + " weight is not loaded");
+    if (w.shape[0] == out_features && w.shape[1] == in_features) return true;
+    LLM_CHECK_WITH_INFO(w.shape[0] == in_features && w.shape[1] == out_features,
+                        std::string(name) + " weight has the wrong shape");
+    return false;
+}
+
+}  // namespace
+
+template <typename T>
+LlamaContextDecoderLayer<T>::LlamaContextDecoderLayer(int head_num, int kv_head_num, int head_size, int inter_size,
+                                                      const LLaMAAttentionStaticParams& attn_params,
+                                                      float rmsnorm_eps, BaseAllocator* allocator)
+    : head_num_(head_num),
+      kv_head_num_(kv_head_num),
+      head_size_(head_size),
+      inter_size_(inter_size),
+      hidden_(head_num * head_size),
+      attn_params_(attn_params),
+      eps_(rmsnorm_eps),
+      allocator_(allocator) {
+    LLM_CHECK_WITH_INFO(allocator != nullptr, "the layer needs an allocator for its buffers");
+    LLM_CHECK_WITH_INFO(head_num > 0 && kv_head_num > 0 && head_num % kv_head_num == 0 && head_size > 0 && inter_size > 0,
+                        "inconsistent layer dimensions");
+    gemm_.reset(new isp_layers::GemmEngine(allocator));
+}
+
+template <typename T>
+LlamaContextDecoderLayer<T>::~LlamaContextDecoderLayer() {
+    freeBuf();
+}
+
+template <typename T>
+size_t LlamaContextDecoderLayer<T>::workspaceBytes(const LLaMAAttentionDynParams& d) const {
+    const size_t tokens = d.num_tokens, b = d.batch_size, q = d.max_q_len, k = d.max_k_len, hs = head_size_;
+    const size_t elems = tokens * (head_num_ + 2 * kv_head_num_) * hs + b * head_num_ * q * hs +
+                         2 * b * head_num_ * k * hs + b * head_num_ * q * k + b * head_num_ * q * hs +
+                         tokens * head_num_ * hs + tokens * 2 * inter_size_ + tokens * inter_size_;
+    return elems * sizeof(T);
+}
+
+template <typename T>
+void LlamaContextDecoderLayer<T>::allocForForward(const LLaMAAttentionDynParams& d) {
+    freeBuf();
+    const size_t tokens = d.num_tokens, b = d.batch_size, q = d.max_q_len, k = d.max_k_len, hs = head_size_;
+    auto take = [this](size_t elems) {
+        return static_cast<T*>(allocator_->UnifyMalloc(nullptr, elems * sizeof(T), false));
+    };
+    qkv_buf_ = take(tokens * (head_num_ + 2 * kv_head_num_) * hs);
+    q_buf_ = take(b * head_num_ * q * hs);
+    k_all_ = take(b * head_num_ * k * hs);
+    v_all_ = take(b * head_num_ * k * hs);
+    scores_ = take(b * head_num_ * q * k);
+    ctx_ = take(b * head_num_ * q * hs);
+    ctx_packed_ = take(tokens * head_num_ * hs);
+    gate_up_ = take(tokens * 2 * inter_size_);
+    act_ = take(tokens * inter_size_);
+    // padded positions of q (and the k / v rows past a sequence's context) are never written by the
+    // kernels; they only meet zero probabilities or discarded rows, but must not hold NaN patterns
+    CHECK(hipMemsetAsync(q_buf_, 0, b * head_num_ * q * hs * sizeof(T), nullptr));
+    CHECK(hipMemsetAsync(k_all_, 0, b * head_num_ * k * hs * sizeof(T), nullptr));
+    CHECK(hipMemsetAsync(v_all_, 0, b * head_num_ * k * hs * sizeof(T), nullptr));
+    allocated_ = d;
+}
+
+template <typename T>
+void LlamaContextDecoderLayer<T>::freeBuf() {
+    T** all[] = {&qkv_buf_, &q_buf_, &k_all_, &v_all_, &scores_, &ctx_, &ctx_packed_, &gate_up_, &act_};
+    for (T** p : all) {
+        if (*p) allocator_->UnifyFree(*p, false);
+        *p = nullptr;
+    }
+    allocated_ = LLaMAAttentionDynParams();
+}
+
+template <typename T>
+void LlamaContextDecoderLayer<T>::forward(TensorMap& inputs, LlamaLayerWeight<T>& weights,
+                                          LayerNormWeight<T>& next_attn_norm, TensorMap& outputs,
+                                          const LLaMAAttentionDynParams& dyn) {
+    TensorWrapper<T>* decoder_input = as<T>(inputs["decoder_input"], "decoder_input");
+    TensorWrapper<T>* residual = as<T>(inputs["decoder_residual"], "decoder_residual");
+    TensorWrapper<int>* padding_offset = as<int>(inputs["padding_offset"], "padding_offset");
+    TensorWrapper<int>* history_length = as<int>(inputs["history_length"], "history_length");
+    TensorWrapper<int>* input_length = as<int>(inputs["input_length"], "input_length");
+    TensorWrapper<int>* context_length = as<int>(inputs["context_length"], "context_length");
+    TensorWrapper<int>* layer_id = as<int>(inputs["layer_id"], "layer_id");
+    TensorWrapper<T>* decoder_output = as<T>(outputs["decoder_output"], "decoder_output");
+    TensorWrapper<T>* k_cache = as<T>(outputs["all_k_cache"], "all_k_cache");
+    TensorWrapper<T>* v_cache = as<T>(outputs["all_v_cache"], "all_v_cache");
+
+    const int tokens = dyn.num_tokens, batch = dyn.batch_size, max_q = dyn.max_q_len, max_k = dyn.max_k_len;
+    const int hs = head_size_, heads = head_num_ + 2 * kv_head_num_;
+    LLM_CHECK_WITH_INFO(decoder_input->shape.size() == 2 && decoder_input->shape[0] == tokens &&
+                            decoder_input->shape[1] == hidden_,
+                        "decoder_input should be [num_tokens, hidden]");
+    LLM_CHECK_WITH_INFO(residual->shape == decoder_input->shape && decoder_output->shape == decoder_input->shape,
+                        "decoder_residual / decoder_output should match decoder_input");
+    LLM_CHECK_WITH_INFO(padding_offset->shape.size() == 2 && padding_offset->shape[0] == batch &&
+                            padding_offset->shape[1] == max_q,
+                        "padding_offset should be [batch, max_q_len]");
+    LLM_CHECK_WITH_INFO(history_length->shape[0] == batch && input_length->shape[0] == batch &&
+                            context_length->shape[0] == batch,
+                        "length tensors should hold one entry per sequence");
+    LLM_CHECK_WITH_INFO(k_cache->shape.size() == 5 && k_cache->shape[3] >= max_k, "KV cache shorter than max_k_len");
+    LLM_CHECK_WITH_INFO(next_attn_norm.gamma != nullptr && weights.ffn_norm_weight.gamma != nullptr,
+                        "norm weights are not loaded");
+    if (tokens == 0) return;
+    if (dyn.num_tokens > allocated_.num_tokens || dyn.batch_size > allocated_.batch_size ||
+        dyn.max_q_len != allocated_.max_q_len || dyn.max_k_len != allocated_.max_k_len)
+        allocForForward(dyn);
+
+    const hipDataType lt = isp_layers::LtType<T>::value;
+    const DataType dt = getTensorType<T>();
+    auto& attn = weights.self_attn_weight;
+    auto& ffn = weights.ffn_weight;
+
+    // 1. fused QKV projection: [tokens, hidden] x Wqkv -> [tokens, heads, hs]   (linear.cu:7)
+    const bool qkv_oi = stored_out_in(attn.qkv, heads * hs, hidden_, "qkv");
+    gemm_->matmul(lt, decoder_input->data, attn.qkv.data, qkv_buf_, tokens, heads * hs, hidden_, qkv_oi, hidden_,
+                  qkv_oi ? hidden_ : heads * hs, heads * hs);
+    // 2. bias + RoPE + transpose / re-pad of q, and k, v straight into the cache
+    TensorWrapper<T> qkv_t(GPU, dt, {tokens, heads, hs}, qkv_buf_);
+    TensorWrapper<T> q_t(GPU, dt, {batch, head_num_, max_q, hs}, q_buf_);
+    launchAddFusedQKVBiasTransposeRoPEAndConcatKV(&q_t, &qkv_t, attn.qkv, padding_offset, history_length,
+                                                  input_length, layer_id, k_cache, v_cache, attn_params_);
+    // 3. cache -> k, v of every query head over the whole context (GQA broadcast)
+    TensorWrapper<T> k_all_t(GPU, dt, {batch, head_num_, max_k, hs}, k_all_);
+    TensorWrapper<T> v_all_t(GPU, dt, {batch, head_num_, max_k, hs}, v_all_);
+    launchRepeatKVCache(k_cache, v_cache, context_length, layer_id, &k_all_t, &v_all_t);
+    // 4. attention: scores = q k^T, masked softmax, ctx = p v   (batched GEMMs, linear.cu:67-109)
+    const int bh = batch * head_num_;
+    gemm_->matmul(lt, q_buf_, k_all_, scores_, max_q, max_k, hs, true, hs, hs, max_k, bh, (long long)max_q * hs,
+                  (long long)max_k * hs, (long long)max_q * max_k);
+    hipLaunchKernelGGL((isp_layers::masked_scaled_softmax<T>), dim3((unsigned)max_q, (unsigned)head_num_, (unsigned)batch),
+                       dim3(256), 0, nullptr, scores_, history_length->data, input_length->data, context_length->data,
+                       head_num_, max_q, max_k, 1.0f / std::sqrt((float)hs));
+    CHECK(hipGetLastError());
+    gemm_->matmul(lt, scores_, v_all_, ctx_, max_q, hs, max_k, false, max_k, hs, hs, bh, (long long)max_q * max_k,
+                  (long long)max_k * hs, (long long)max_q * hs);
+    // 5. [batch, heads, max_q, hs] -> packed [tokens, heads, hs]
+    TensorWrapper<T> ctx_t(GPU, dt, {batch, head_num_, max_q, hs}, ctx_);
+    TensorWrapper<T> packed_t(GPU, dt, {tokens, head_num_, hs}, ctx_packed_);
+    launchTransposeOutRemovePadding(&ctx_t, padding_offset, &packed_t);
+    // 6. output projection into decoder_input's storage (its contents are no longer needed)   (linear.cu:8)
+    const bool o_oi = stored_out_in(attn.output, hidden_, hidden_, "attention output");
+    gemm_->matmul(lt, ctx_packed_, attn.output.data, decoder_input->data, tokens, hidden_, hidden_, o_oi, hidden_,
+                  hidden_, hidden_);
+    // 7. residual += attn (+ bias); decoder_input := RMSNorm by ffn_norm
+    launchFusedAddBiasResidualRMSNorm(residual, decoder_input, attn.output, weights.ffn_norm_weight.gamma, eps_);
+    // 8. gate / up projection -> [tokens, 2, inter]   (linear.cu:14)
+    const bool gu_oi = stored_out_in(ffn.gateAndup, 2 * inter_size_, hidden_, "gate/up");
+    gemm_->matmul(lt, decoder_input->data, ffn.gateAndup.data, gate_up_, tokens, 2 * inter_size_, hidden_, gu_oi,
+                  hidden_, gu_oi ? hidden_ : 2 * inter_size_, 2 * inter_size_);
+    // 9. SwiGLU
+    TensorWrapper<T> gate_up_t(GPU, dt, {tokens, 2, inter_size_}, gate_up_);
+    TensorWrapper<T> act_t(GPU, dt, {tokens, inter_size_}, act_);
+    launchAct(&gate_up_t, &act_t);
+    // 10. down projection   (linear.cu:15)
+    const bool down_oi = stored_out_in(ffn.down, hidden_, inter_size_, "down");
+    gemm_->matmul(lt, act_, ffn.down.data, decoder_output->data, tokens, hidden_, inter_size_, down_oi, inter_size_,
+                  down_oi ? inter_size_ : hidden_, hidden_);
+    // 11. residual += ffn (+ bias); decoder_output := RMSNorm by the next layer's attention norm
+    launchFusedAddBiasResidualRMSNorm(residual, decoder_output, ffn.down, next_attn_norm.gamma, eps_);
+}
+
+template class LlamaContextDecoderLayer<float>;
+template class LlamaContextDecoderLayer<half>;

@@ -1,0 +1,209 @@
+// Call site of the C++ context-decoder layer (LlamaContextDecoderLayer over TensorMap / LlamaLayerWeight /
+// BaseAllocator).  The program builds a small ragged batch, runs one layer, and writes every operand and
+// result as raw little-endian float32 files into a directory; tests/test_cpp_context_layer.py reads them
+// back and checks the results against an independent float64 implementation of the same layer.  A second
+// case checks, inside the program, that two turns through the KV cache reproduce one long prefill.
+//
+//   test_context_layer <f32|f16> <directory> [head_num kv_head_num head_size inter_size]
+#include <cstdio>
+#include <numeric>
+#include <string>
+
+#include "src/kernels/cal_paddingoffset.h"
+#include "src/kernels/rmsnorm.h"
+#include "src/layers/decoder/context_decoder_layer.h"
+#include "src/memory/allocator/hip_allocator.h"
+#include "test_util.h"
+
+template <typename T>
+static void dump(const std::string& dir, const char* name, const T* device, size_t n) {
+    using S = typename Host<T>::Store;
+    auto h = to_host(reinterpret_cast<const S*>(device), n);
+    std::vector<float> f(n);
+    for (size_t i = 0; i < n; i++) f[i] = Host<T>::from(h[i]);
+    const std::string path = dir + "/" + name + ".bin";
+    FILE* fp = std::fopen(path.c_str(), "wb");
+    if (!fp || std::fwrite(f.data(), sizeof(float), n, fp) != n) {
+        std::printf("cannot write %s\n", path.c_str());
+        std::exit(2);
+    }
+    std::fclose(fp);
+}
+
+template <typename T>
+struct Batch {
+    int batch, max_q, tokens, max_k;
+    int *lens, *hist, *ctx, *padding_offset, *cum;
+    Batch(const std::vector<int>& l, const std::vector<int>& h, int max_q_len) : batch((int)l.size()), max_q(max_q_len) {
+        tokens = std::accumulate(l.begin(), l.end(), 0);
+        std::vector<int> c(batch);
+        max_k = 0;
+        for (int b = 0; b < batch; b++) {
+            c[b] = l[b] + h[b];
+            max_k = std::max(max_k, c[b]);
+        }
+        lens = to_device(l);
+        hist = to_device(h);
+        ctx = to_device(c);
+        padding_offset = to_device(std::vector<int>((size_t)batch * max_q, 0));
+        cum = to_device(std::vector<int>(batch + 1, 0));
+        TensorWrapper<int> po(Device::GPU, getTensorType<int>(), {batch, max_q}, padding_offset);
+        TensorWrapper<int> cs(Device::GPU, getTensorType<int>(), {batch + 1}, cum);
+        TensorWrapper<int> il(Device::GPU, getTensorType<int>(), {batch}, lens);
+        launchCalPaddingoffset(&po, &cs, &il);
+    }
+};
+
+// Runs one layer on `rows` (packed [tokens, hidden], storage type); returns through the device buffers.
+template <typename T>
+static void run_layer(LlamaContextDecoderLayer<T>& layer, LlamaLayerWeight<T>& w, LayerNormWeight<T>& next,
+                      Batch<T>& bt, T* residual, T* normed, T* out, T* k_cache, T* v_cache, int layers, int kv_heads,
+                      int max_seq, int head_size, int hidden, int layer_index) {
+    const DataType dt = getTensorType<T>();
+    CHECK(hipMemcpy(normed, residual, (size_t)bt.tokens * hidden * sizeof(T), hipMemcpyDeviceToDevice));
+    TensorWrapper<T> in(Device::GPU, dt, {bt.tokens, hidden}, normed);
+    launchRMSNorm(&in, w.attn_norm_weight, 1e-5f);
+    TensorWrapper<T> res(Device::GPU, dt, {bt.tokens, hidden}, residual);
+    TensorWrapper<T> o(Device::GPU, dt, {bt.tokens, hidden}, out);
+    TensorWrapper<int> po(Device::GPU, getTensorType<int>(), {bt.batch, bt.max_q}, bt.padding_offset);
+    TensorWrapper<int> hl(Device::GPU, getTensorType<int>(), {bt.batch}, bt.hist);
+    TensorWrapper<int> il(Device::GPU, getTensorType<int>(), {bt.batch}, bt.lens);
+    TensorWrapper<int> cl(Device::GPU, getTensorType<int>(), {bt.batch}, bt.ctx);
+    int layer_value = layer_index;
+    TensorWrapper<int> lid(Device::CPU, getTensorType<int>(), {1}, &layer_value);
+    TensorWrapper<T> kc(Device::GPU, dt, {layers, bt.batch, kv_heads, max_seq, head_size}, k_cache);
+    TensorWrapper<T> vc(Device::GPU, dt, {layers, bt.batch, kv_heads, max_seq, head_size}, v_cache);
+    TensorMap inputs{{"decoder_input", &in}, {"decoder_residual", &res}, {"padding_offset", &po},
+                     {"history_length", &hl}, {"input_length", &il}, {"context_length", &cl}, {"layer_id", &lid}};
+    TensorMap outputs{{"decoder_output", &o}, {"all_k_cache", &kc}, {"all_v_cache", &vc}};
+    LLaMAAttentionDynParams dyn;
+    dyn.batch_size = bt.batch;
+    dyn.num_tokens = bt.tokens;
+    dyn.max_q_len = bt.max_q;
+    dyn.max_k_len = bt.max_k;
+    dyn.num_layers = layers;
+    layer.forward(inputs, w, next, outputs, dyn);
+    CHECK(hipDeviceSynchronize());
+}
+
+template <typename T>
+static int run(const std::string& dir, int head_num, int kv_heads, int head_size, int inter) {
+    using S = typename Host<T>::Store;
+    const int hidden = head_num * head_size, layers = 2, max_seq = 32, max_q = 16;
+    HipAllocator allocator;
+    LLaMAAttentionStaticParams params;
+    params.rotary_embedding_dim = head_size;
+    LlamaLayerWeight<T> w(head_num, kv_heads, head_size, inter, getWeightType<T>(), /*attn_bias=*/true);
+    w.loadWeights();
+    std::mt19937 gen(17);
+    LayerNormWeight<T> next;
+    next.gamma = (T*)to_device(randn<T>(hidden, 0.25f, gen, 1.0f));
+    LlamaContextDecoderLayer<T> layer(head_num, kv_heads, head_size, inter, params, 1e-5f, &allocator);
+
+    // ---- case 1: ragged batch, checked by the Python side against float64
+    const std::vector<int> lens = {16, 5, 11}, hist = {0, 0, 0};
+    Batch<T> bt(lens, hist, max_q);
+    auto rows = randn<T>((size_t)bt.tokens * hidden, 1.0f, gen);
+    T* residual = (T*)to_device(rows);
+    T* normed = (T*)to_device(std::vector<S>(rows.size()));
+    T* out = (T*)to_device(std::vector<S>(rows.size()));
+    const size_t cache_elems = (size_t)layers * bt.batch * kv_heads * max_seq * head_size;
+    T* k_cache = (T*)to_device(std::vector<S>(cache_elems));
+    T* v_cache = (T*)to_device(std::vector<S>(cache_elems));
+    dump<T>(dir, "residual_in", residual, rows.size());
+    run_layer(layer, w, next, bt, residual, normed, out, k_cache, v_cache, layers, kv_heads, max_seq, head_size, hidden, 1);
+    const int qkv_out = (head_num + 2 * kv_heads) * head_size;
+    dump<T>(dir, "attn_norm", w.attn_norm_weight.gamma, hidden);
+    dump<T>(dir, "ffn_norm", w.ffn_norm_weight.gamma, hidden);
+    dump<T>(dir, "next_norm", next.gamma, hidden);
+    dump<T>(dir, "qkv_weight", w.self_attn_weight.qkv.data, (size_t)qkv_out * hidden);
+    dump<T>(dir, "qkv_bias", w.self_attn_weight.qkv.bias, qkv_out);
+    dump<T>(dir, "o_weight", w.self_attn_weight.output.data, (size_t)hidden * hidden);
+    dump<T>(dir, "o_bias", w.self_attn_weight.output.bias, hidden);
+    dump<T>(dir, "gate_up_weight", w.ffn_weight.gateAndup.data, (size_t)2 * inter * hidden);
+    dump<T>(dir, "down_weight", w.ffn_weight.down.data, (size_t)hidden * inter);
+    dump<T>(dir, "residual_out", residual, rows.size());
+    dump<T>(dir, "decoder_output", out, rows.size());
+    dump<T>(dir, "k_cache", k_cache, cache_elems);
+    dump<T>(dir, "v_cache", v_cache, cache_elems);
+
+    // ---- case 2: 9 tokens, then 7 more with history 9, must equal one 16-token prefill
+    auto x = randn<T>((size_t)16 * hidden, 1.0f, gen);
+    auto once = [&](const std::vector<int>& l, const std::vector<int>& h, const S* src, size_t n_tokens, T* kc, T* vc,
+                    std::vector<S>& res_out, std::vector<S>& next_out) {
+        Batch<T> b1(l, h, max_q);
+        std::vector<S> part(src, src + n_tokens * hidden);
+        T* r = (T*)to_device(part);
+        T* nrm = (T*)to_device(std::vector<S>(part.size()));
+        T* o = (T*)to_device(std::vector<S>(part.size()));
+        run_layer(layer, w, next, b1, r, nrm, o, kc, vc, 1, kv_heads, max_seq, head_size, hidden, 0);
+        res_out = to_host((S*)r, part.size());
+        next_out = to_host((S*)o, part.size());
+    };
+    const size_t one_cache = (size_t)kv_heads * max_seq * head_size;
+    T* kc_a = (T*)to_device(std::vector<S>(one_cache));
+    T* vc_a = (T*)to_device(std::vector<S>(one_cache));
+    T* kc_b = (T*)to_device(std::vector<S>(one_cache));
+    T* vc_b = (T*)to_device(std::vector<S>(one_cache));
+    std::vector<S> r_all, o_all, r1, o1, r2, o2;
+    once({16}, {0}, x.data(), 16, kc_a, vc_a, r_all, o_all);
+    once({9}, {0}, x.data(), 9, kc_b, vc_b, r1, o1);
+    once({7}, {9}, x.data() + (size_t)9 * hidden, 7, kc_b, vc_b, r2, o2);
+    r1.insert(r1.end(), r2.begin(), r2.end());
+    o1.insert(o1.end(), o2.begin(), o2.end());
+    double scale_r = 0, scale_o = 0, err_r = 0, err_o = 0;
+    for (size_t i = 0; i < r_all.size(); i++) {
+        scale_r = std::max(scale_r, std::fabs((double)Host<T>::from(r_all[i])));
+        scale_o = std::max(scale_o, std::fabs((double)Host<T>::from(o_all[i])));
+        err_r = std::max(err_r, std::fabs((double)Host<T>::from(r_all[i]) - Host<T>::from(r1[i])));
+        err_o = std::max(err_o, std::fabs((double)Host<T>::from(o_all[i]) - Host<T>::from(o1[i])));
+    }
+    const double tol = std::is_same<T, float>::value ? 2e-4 : 2e-2;
+    EXPECT(err_r <= tol * scale_r, "two turns: residual differs by %g (scale %g)", err_r, scale_r);
+    EXPECT(err_o <= tol * scale_o, "two turns: output differs by %g (scale %g)", err_o, scale_o);
+    auto ka = to_host((S*)kc_a, one_cache), kb = to_host((S*)kc_b, one_cache);
+    double err_k = 0;
+    for (size_t i = 0; i < ka.size(); i++) err_k = std::max(err_k, std::fabs((double)Host<T>::from(ka[i]) - Host<T>::from(kb[i])));
+    EXPECT(err_k <= tol * 8.0, "two turns: cached keys differ by %g", err_k);
+
+    // ---- the layer rejects tensors that do not fit
+    {
+        Batch<T> b2(lens, hist, max_q);
+        T* r = (T*)to_device(rows);
+        TensorWrapper<T> bad(Device::GPU, getTensorType<T>(), {bt.tokens, hidden + 1}, r);
+        TensorWrapper<T> good(Device::GPU, getTensorType<T>(), {bt.tokens, hidden}, r);
+        TensorWrapper<int> po(Device::GPU, getTensorType<int>(), {bt.batch, bt.max_q}, b2.padding_offset);
+        TensorWrapper<int> hl(Device::GPU, getTensorType<int>(), {bt.batch}, b2.hist);
+        int lv = 0;
+        TensorWrapper<int> lid(Device::CPU, getTensorType<int>(), {1}, &lv);
+        TensorWrapper<T> kc(Device::GPU, getTensorType<T>(), {layers, bt.batch, kv_heads, max_seq, head_size}, k_cache);
+        TensorMap inputs{{"decoder_input", &bad}, {"decoder_residual", &good}, {"padding_offset", &po}, {"history_length", &hl},
+                         {"input_length", &hl}, {"context_length", &hl}, {"layer_id", &lid}};
+        TensorMap outputs{{"decoder_output", &good}, {"all_k_cache", &kc}, {"all_v_cache", &kc}};
+        LLaMAAttentionDynParams dyn;
+        dyn.batch_size = bt.batch, dyn.num_tokens = bt.tokens, dyn.max_q_len = max_q, dyn.max_k_len = 16;
+        EXPECT(throws([&] { layer.forward(inputs, w, next, outputs, dyn); }), "a mis-shaped decoder_input must throw");
+        TensorMap missing{{"decoder_input", &good}};
+        EXPECT(throws([&] { layer.forward(missing, w, next, outputs, dyn); }), "a missing input must throw");
+    }
+    std::printf("context layer %s: %d tokens, hidden %d, %d/%d heads x %d, inter %d: %s\n",
+                std::is_same<T, float>::value ? "f32" : "f16", bt.tokens, hidden, head_num, kv_heads, head_size, inter,
+                g_failures ? "FAILED" : "passed");
+    return g_failures;
+}
+
+int main(int argc, char** argv) {
+    if (argc < 3) {
+        std::printf("usage: test_context_layer <f32|f16> <directory> [head_num kv_head_num head_size inter_size]\n");
+        return 2;
+    }
+    const std::string type = argv[1], dir = argv[2];
+    const int head_num = argc > 6 ? std::atoi(argv[3]) : 2, kv = argc > 6 ? std::atoi(argv[4]) : 2;
+    const int hs = argc > 6 ? std::atoi(argv[5]) : 128, inter = argc > 6 ? std::atoi(argv[6]) : 512;
+    try {
+        return type == "f16" ? run<half>(dir, head_num, kv, hs, inter) : run<float>(dir, head_num, kv, hs, inter);
+    } catch (const std::exception& e) {
+        std::printf("exception: %s\n", e.what());
+        return 1;
+    }
+}
