@@ -3,8 +3,10 @@
  * per-layer kernels.
  *
  * This is the drop-in boundary: every entry point takes raw device pointers, plain integers and a
- * HIP stream, launches hand-written HIP kernels asynchronously on that stream, allocates nothing,
- * keeps no state and returns 0 or a negative isp_status.  The C++ `launch*` templates declared
+ * HIP stream, launches hand-written HIP kernels asynchronously on that stream, allocates nothing
+ * and returns 0 or a negative isp_status.  The library keeps no state between calls except the
+ * process-wide tuning knobs of isp_tuning_set (atomic; they select among kernel variants with
+ * identical results, and nothing sets them unless the caller does).  The C++ `launch*` templates declared
  * under include/src/kernels/ (same names and parameter lists as the reference's) are thin shims
  * over these functions; a binding from any other language needs only this header.
  *
@@ -261,7 +263,8 @@ int isp_repeat_kv_cache_f16(const void* k_cache, const void* v_cache, void* k_ds
  *   copy bandwidth the machine actually reaches.
  * isp_tuning_set: overrides a launch heuristic process-wide (0 restores the automatic choice) and
  *   returns the previous value, or ISP_ERR_BAD_SHAPE for an unknown knob.  For benchmark sweeps;
- *   results never depend on the knobs, only speed does.
+ *   results never depend on the knobs, only speed does.  Thread-safe (each knob is an atomic that a
+ *   launcher reads once per call); a serving process has no reason to call it.
  */
 int isp_calibration_copy(void* dst, const void* src, size_t bytes, isp_stream_t stream);
 /* isp_norm_launch_config: which instantiation isp_rmsnorm_* / isp_fused_add_bias_residual_rmsnorm_*

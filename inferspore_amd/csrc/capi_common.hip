@@ -1,6 +1,8 @@
 // Library-wide pieces of the C ABI: status strings, launch-error bookkeeping, device check.
 #include <string.h>
 
+#include <atomic>
+
 #include "isp_common.h"
 
 namespace isp {
@@ -13,23 +15,30 @@ int note_launch(hipError_t e) {
     return ISP_ERR_LAUNCH;
 }
 
-static int g_tuning[ISP_TUNE_COUNT] = {0};
+// Process-wide launch-heuristic overrides.  Relaxed atomics: a launcher reads each knob once per call,
+// so a thread that sets a knob while others launch changes which variant later launches pick (never
+// their results), without a data race.
+static std::atomic<int> g_tuning[ISP_TUNE_COUNT];
 
 int resident_waves() {
     constexpr int kMaxDevices = 64;
-    static int cached[kMaxDevices] = {0};  // written with the same value by every thread
+    static std::atomic<int> cached[kMaxDevices];  // every thread stores the same value
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 256 * 32;
-    if (cached[dev] == 0) {
+    int waves = cached[dev].load(std::memory_order_relaxed);
+    if (waves == 0) {
         int cus = 0;
         if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
             cus = 256;
-        cached[dev] = cus * 32;  // 4 SIMDs x 8 wavefronts per compute unit
+        waves = cus * 32;  // 4 SIMDs x 8 wavefronts per compute unit
+        cached[dev].store(waves, std::memory_order_relaxed);
     }
-    return cached[dev];
+    return waves;
 }
 
-int tuning(int knob) { return (knob >= 0 && knob < ISP_TUNE_COUNT) ? g_tuning[knob] : 0; }
+int tuning(int knob) {
+    return (knob >= 0 && knob < ISP_TUNE_COUNT) ? g_tuning[knob].load(std::memory_order_relaxed) : 0;
+}
 
 }  // namespace isp
 
@@ -37,9 +46,7 @@ extern "C" {
 
 int isp_tuning_set(int knob, int value) {
     if (knob < 0 || knob >= ISP_TUNE_COUNT) return ISP_ERR_BAD_SHAPE;
-    const int old = isp::g_tuning[knob];
-    isp::g_tuning[knob] = value;
-    return old;
+    return isp::g_tuning[knob].exchange(value, std::memory_order_relaxed);
 }
 
 const char* isp_version(void) { return "inferspore_amd 0.1 (gfx950)"; }

@@ -3,7 +3,12 @@
 // reference's launcher does (cited per function), keeps the reference's own argument checks, and
 // launches on the null stream like the reference.  A non-zero status from the C ABI becomes the
 // same std::runtime_error the reference's LLM_CHECK raises.
+#include <atomic>
+#include <cstdlib>
+#include <cstring>
+
 #include "inferspore_amd.h"
+#include "inferspore_amd_shims.h"
 #include "src/kernels/act_kernel.h"
 #include "src/kernels/cal_paddingoffset.h"
 #include "src/kernels/concat_past_kv.h"
@@ -45,11 +50,24 @@ struct Abi<half> {
     static constexpr auto repeat_kv = isp_repeat_kv_cache_f16;
 };
 
+std::atomic<int>& literal_bias_setting() {
+    static std::atomic<int> setting([] {
+        const char* env = std::getenv("ISP_SHIMS_REFERENCE_LITERAL_BIAS");
+        return (env != nullptr && std::strcmp(env, "1") == 0) ? 1 : 0;
+    }());
+    return setting;
+}
+
 inline void expect_ok(int status, const char* what) {
     LLM_CHECK_WITH_INFO(status == ISP_OK, std::string(what) + ": " + isp_strerror(status));
 }
 
 }  // namespace
+
+namespace isp_shims {
+bool setReferenceLiteralBias(bool on) { return literal_bias_setting().exchange(on ? 1 : 0) != 0; }
+bool referenceLiteralBias() { return literal_bias_setting().load() != 0; }
+}  // namespace isp_shims
 
 // reference: src/kernels/input_embedding.cu:25-45 (token count and hidden size from output->shape,
 // the shape check at :35)
@@ -87,8 +105,9 @@ void launchFusedAddBiasResidualRMSNorm(TensorWrapper<T>* residual, TensorWrapper
                                        BaseWeight<T>& norm, T* scale, float eps) {
     const int tokens = decoder_out->shape[0];
     const int hidden = decoder_out->shape[1];
+    const unsigned flags = isp_shims::referenceLiteralBias() ? ISP_NORM_RESIDUAL_EXCLUDES_BIAS : 0u;
     expect_ok(Abi<T>::fused_norm(residual->data, decoder_out->data, norm.bias, scale, eps, tokens,
-                                 hidden, 0u, nullptr),
+                                 hidden, flags, nullptr),
               "launchFusedAddBiasResidualRMSNorm");
 }
 
@@ -114,7 +133,8 @@ void launchAddFusedQKVBiasTransposeAndRoPE(TensorWrapper<T>* q_buf, TensorWrappe
     const int head_num = q_buf->shape[1];
     const int seq_len = q_buf->shape[2];
     const int kv_head_num = (qkv_head_num - head_num) / 2;
-    expect_ok(Abi<T>::qkv(q_buf->data, k_buf->data, v_buf->data, QKV->data, qkv.bias,
+    const T* bias = isp_shims::referenceLiteralBias() ? nullptr : qkv.bias;
+    expect_ok(Abi<T>::qkv(q_buf->data, k_buf->data, v_buf->data, QKV->data, bias,
                           padding_offset->data, history_length->data, input_length->data,
                           batch_size, seq_len, token_num, head_num, kv_head_num, head_size,
                           params.rotary_embedding_dim, params.rotary_embedding_base,
@@ -147,8 +167,9 @@ void launchAddFusedQKVBiasTransposeRoPEAndConcatKV(TensorWrapper<T>* q_buf, Tens
                         "k / v cache extents should match the qkv buffer's");
     const int layer = layer_id->getVal();
     LLM_CHECK_WITH_INFO(layer >= 0 && layer < k_cache->shape[0], "layer id outside the cache");
+    const T* bias = isp_shims::referenceLiteralBias() ? nullptr : qkv.bias;
     expect_ok(Abi<T>::qkv_append(q_buf->data, nullptr, nullptr, k_cache->data, v_cache->data, layer,
-                                 k_cache->shape[3], QKV->data, qkv.bias, padding_offset->data,
+                                 k_cache->shape[3], QKV->data, bias, padding_offset->data,
                                  history_length->data, input_length->data, batch_size, seq_len,
                                  token_num, head_num, kv_head_num, head_size,
                                  params.rotary_embedding_dim, params.rotary_embedding_base, nullptr),

@@ -67,7 +67,7 @@ __global__ __launch_bounds__(kBlock) void swiglu_generic(const T* in, T* out, si
         const size_t gate = i + t * inter;
         const float a = Elem<T>::to_f32(in[gate]);
         const float b = Elem<T>::to_f32(in[gate + inter]);
-        out[i] = Elem<T>::from_f32(silu_exact(a) * b);
+        out[i] = Elem<T>::from_f32(silu_for<T>(a) * b);  // same formulation as swiglu_vec: bit-identical
     }
 }
 

@@ -12,7 +12,8 @@ import subprocess
 import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-_SO = os.path.join(_HERE, "libisp_oracle.so")
+# ISP_ORACLE_LIB names another build of the same source (the sanitizer build of `make -C oracle asan`)
+_SO = os.environ.get("ISP_ORACLE_LIB") or os.path.join(_HERE, "libisp_oracle.so")
 
 NORM_RESIDUAL_EXCLUDES_BIAS = 1
 

@@ -4,7 +4,7 @@
 // the known answers those reference programs state.  Unlike the reference's programs, a mismatch
 // fails the process.
 //
-//   test_launch_api <case>      case = embedding | padding | norm | rmsnorm | qkv | act | errors | all
+//   test_launch_api <case>      case = embedding | padding | norm | rmsnorm | qkv | act | bias_modes | errors | all
 #include <hip/hip_runtime.h>
 
 #include <cmath>
@@ -16,6 +16,7 @@
 #include <string>
 #include <vector>
 
+#include "inferspore_amd_shims.h"
 #include "isp_oracle.h"
 #include "src/kernels/act_kernel.h"
 #include "src/kernels/cal_paddingoffset.h"
@@ -227,6 +228,90 @@ void case_qkv() {
     EXPECT(std::memcmp(gv.data(), ev.data(), qn * sizeof(S)) == 0, "v differs from the oracle");
 }
 
+// --------------------------------------------------------------------------- the two bias modes
+// Non-null biases through the launchers, once as the operators' names say (the default) and once as
+// the reference's kernels literally behave (isp_shims::setReferenceLiteralBias): each mode against the
+// oracle run in the same mode, and the two modes must differ exactly where the bias enters.
+template <typename T>
+void case_bias_modes() {
+    using S = typename Host<T>::Store;
+    const bool before = isp_shims::referenceLiteralBias();
+    for (int literal = 0; literal < 2; literal++) {
+        isp_shims::setReferenceLiteralBias(literal != 0);
+        EXPECT(isp_shims::referenceLiteralBias() == (literal != 0), "setting must read back");
+        {   // fused norm: the normalised output includes the bias in both modes, the stored residual only by default
+            const int tokens = 33, hidden = 1024;
+            std::mt19937 gen(21);
+            auto out = randn<T>((size_t)tokens * hidden, 1.f, gen);
+            auto res = randn<T>((size_t)tokens * hidden, 1.f, gen);
+            auto bias = randn<T>(hidden, 0.5f, gen);
+            auto gamma = randn<T>(hidden, 0.25f, gen, 1.0f);
+            S *d_out = to_device(out), *d_res = to_device(res), *d_bias = to_device(bias), *d_gamma = to_device(gamma);
+            TensorWrapper<T> out_t(Device::GPU, getTensorType<T>(), {tokens, hidden}, (T*)d_out);
+            TensorWrapper<T> res_t(Device::GPU, getTensorType<T>(), {tokens, hidden}, (T*)d_res);
+            BaseWeight<T> norm;
+            norm.bias = (T*)d_bias;
+            launchFusedAddBiasResidualRMSNorm(&res_t, &out_t, norm, (T*)d_gamma, 1e-5f);
+            auto res_other = res, out_other = out;
+            const unsigned flags = literal ? ISP_ORACLE_NORM_RESIDUAL_EXCLUDES_BIAS : 0u;
+            if (std::is_same<T, float>::value) {
+                isp_oracle_fused_norm_f32((float*)res.data(), (float*)out.data(), (const float*)bias.data(), (const float*)gamma.data(), 1e-5f, tokens, hidden, flags);
+                isp_oracle_fused_norm_f32((float*)res_other.data(), (float*)out_other.data(), (const float*)bias.data(), (const float*)gamma.data(), 1e-5f, tokens, hidden, flags ^ 1u);
+            } else {
+                isp_oracle_fused_norm_f16((uint16_t*)res.data(), (uint16_t*)out.data(), (const uint16_t*)bias.data(), (const uint16_t*)gamma.data(), 1e-5f, tokens, hidden, flags);
+                isp_oracle_fused_norm_f16((uint16_t*)res_other.data(), (uint16_t*)out_other.data(), (const uint16_t*)bias.data(), (const uint16_t*)gamma.data(), 1e-5f, tokens, hidden, flags ^ 1u);
+            }
+            compare<T>(to_host(d_out, out.size()), out, literal ? "literal mode: normalised output" : "default mode: normalised output");
+            auto got_res = to_host(d_res, res.size());
+            EXPECT(std::memcmp(got_res.data(), res.data(), res.size() * sizeof(S)) == 0, "mode %d: residual differs from the oracle in the same mode", literal);
+            EXPECT(std::memcmp(got_res.data(), res_other.data(), res.size() * sizeof(S)) != 0, "mode %d: residual must differ from the other mode's", literal);
+            CHECK(hipFree(d_out)); CHECK(hipFree(d_res)); CHECK(hipFree(d_bias)); CHECK(hipFree(d_gamma));
+        }
+        {   // QKV: the bias is added by default and ignored in the literal mode
+            const int batch = 2, seq = 9, hn = 32, kvn = 32, hs = 128;
+            const std::vector<int> lens = {9, 4}, hist = {5, 0};
+            const int tokens = 13;
+            std::mt19937 gen(22);
+            auto qkv = randn<T>((size_t)tokens * (hn + 2 * kvn) * hs, 1.f, gen);
+            auto bias = randn<T>((size_t)(hn + 2 * kvn) * hs, 0.5f, gen);
+            std::vector<int> po(batch * seq, 0), cum(batch + 1, 0);
+            isp_oracle_cal_padding_offset(po.data(), cum.data(), lens.data(), batch, seq);
+            int *d_lens = to_device(lens), *d_hist = to_device(hist), *d_po = to_device(po);
+            TensorWrapper<int> po_t(Device::GPU, getTensorType<int>(), {batch, seq}, d_po);
+            TensorWrapper<int> lens_t(Device::GPU, getTensorType<int>(), {batch}, d_lens);
+            TensorWrapper<int> hist_t(Device::GPU, getTensorType<int>(), {batch}, d_hist);
+            const size_t qn = (size_t)batch * hn * seq * hs;
+            const S sentinel = Host<T>::to(-77.f);
+            S *dq = to_device(std::vector<S>(qn, sentinel)), *dk = to_device(std::vector<S>(qn, sentinel)), *dv = to_device(std::vector<S>(qn, sentinel));
+            S *d_qkv = to_device(qkv), *d_bias = to_device(bias);
+            TensorWrapper<T> q_t(Device::GPU, getTensorType<T>(), {batch, hn, seq, hs}, (T*)dq);
+            TensorWrapper<T> k_t(Device::GPU, getTensorType<T>(), {batch, kvn, seq, hs}, (T*)dk);
+            TensorWrapper<T> v_t(Device::GPU, getTensorType<T>(), {batch, kvn, seq, hs}, (T*)dv);
+            TensorWrapper<T> qkv_t(Device::GPU, getTensorType<T>(), {tokens, hn + 2 * kvn, hs}, (T*)d_qkv);
+            BaseWeight<T> w;
+            w.bias = (T*)d_bias;
+            LLaMAAttentionStaticParams params;
+            launchAddFusedQKVBiasTransposeAndRoPE(&q_t, &k_t, &v_t, &qkv_t, w, &po_t, &hist_t, &lens_t, params);
+            std::vector<S> eq(qn, sentinel), ek(qn, sentinel), ev(qn, sentinel);
+            const void* oracle_bias = literal ? nullptr : bias.data();
+            if (std::is_same<T, float>::value)
+                isp_oracle_qkv_rope_f32((float*)eq.data(), (float*)ek.data(), (float*)ev.data(), (const float*)qkv.data(), (const float*)oracle_bias,
+                                        po.data(), hist.data(), lens.data(), batch, seq, tokens, hn, kvn, hs, 128, 10000.f);
+            else
+                isp_oracle_qkv_rope_f16((uint16_t*)eq.data(), (uint16_t*)ek.data(), (uint16_t*)ev.data(), (const uint16_t*)qkv.data(),
+                                        (const uint16_t*)oracle_bias, po.data(), hist.data(), lens.data(), batch, seq, tokens, hn, kvn, hs, 128, 10000.f);
+            auto mag = [](size_t) { return 8.0; };
+            compare<T>(to_host(dq, qn), eq, literal ? "literal mode: q" : "default mode: q", mag);
+            compare<T>(to_host(dk, qn), ek, literal ? "literal mode: k" : "default mode: k", mag);
+            auto gv = to_host(dv, qn);
+            EXPECT(std::memcmp(gv.data(), ev.data(), qn * sizeof(S)) == 0, "mode %d: v differs from the oracle in the same mode", literal);
+            CHECK(hipFree(dq)); CHECK(hipFree(dk)); CHECK(hipFree(dv)); CHECK(hipFree(d_qkv)); CHECK(hipFree(d_bias));
+            CHECK(hipFree(d_lens)); CHECK(hipFree(d_hist)); CHECK(hipFree(d_po));
+        }
+    }
+    isp_shims::setReferenceLiteralBias(before);
+}
+
 // --------------------------------------------------------------------------- swiglu
 template <typename T>
 void case_act() {
@@ -295,6 +380,7 @@ int main(int argc, char** argv) {
         {"rmsnorm", [] { case_rmsnorm<float>(); case_rmsnorm<half>(); }},
         {"qkv", [] { case_qkv<float>(); case_qkv<half>(); }},
         {"act", [] { case_act<float>(); case_act<half>(); }},
+        {"bias_modes", [] { case_bias_modes<float>(); case_bias_modes<half>(); }},
         {"errors", [] { case_errors(); }},
     };
     for (auto& kv : cases) {

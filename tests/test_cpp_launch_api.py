@@ -14,7 +14,7 @@ LAUNCH_LIB = os.path.join(ROOT, "inferspore_amd", "lib", "libinferspore_launch.s
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("case", ["embedding", "padding", "norm", "rmsnorm", "qkv", "act", "errors"])
+@pytest.mark.parametrize("case", ["embedding", "padding", "norm", "rmsnorm", "qkv", "act", "bias_modes", "errors"])
 def test_launch_api_case(case):
     assert os.path.exists(EXE), "build/bin/test_launch_api is missing: run python -m inferspore_amd.build"
     print("[case] test_launch_api " + case, flush=True)

@@ -135,6 +135,32 @@ def test_swiglu_every_unroll_and_store_kind(isp, oracle, dtype):
         assert np.array_equal(with_knobs({capi.TUNE_SWIGLU_UNROLL: unroll, capi.TUNE_SWIGLU_STORE: store}, run), base)
 
 
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+def test_swiglu_vector_and_scalar_kernels_agree_bit_for_bit(isp, dtype):
+    """An input at a 16-byte boundary takes the vector kernel, the same values one element further on take
+    the scalar one; a caller must not see the difference, in either precision."""
+    tokens, inter = 37, 1408
+    x = swiglu_inputs(tokens, inter, dtype, seed=17) * dtype(3)
+    td = NP2T[dtype]
+    aligned_out = torch.zeros((tokens, inter), dtype=td, device="cuda")
+    isp.act(dev(x), aligned_out)
+    flat = torch.zeros(x.size + 1, dtype=td, device="cuda")
+    flat[1:] = dev(x).view(-1)
+    shifted_in = flat[1:].view(tokens, 2, inter)
+    assert shifted_in.data_ptr() % 16 != 0
+    for out_shift in (0, 1):
+        say("swiglu %s misaligned input, output shift %d" % (dtype.__name__, out_shift))
+        out_flat = torch.zeros(tokens * inter + 1, dtype=td, device="cuda")
+        out = out_flat[out_shift:out_shift + tokens * inter].view(tokens, inter)
+        isp.act(shifted_in, out)
+        assert torch.equal(out, aligned_out)
+    say("swiglu %s aligned input, misaligned output" % dtype.__name__)
+    out_flat = torch.zeros(tokens * inter + 1, dtype=td, device="cuda")
+    out = out_flat[1:].view(tokens, inter)
+    isp.act(dev(x), out)
+    assert torch.equal(out, aligned_out)
+
+
 def test_calibration_copy(isp):
     from inferspore_amd import capi
     lib = capi.lib()
