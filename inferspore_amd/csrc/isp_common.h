@@ -222,6 +222,27 @@ struct Elem<__half> {
     }
 };
 
+// Unsigned division by a launch constant without the integer-divide expansion: q = floor(p / d) from
+// one multiply-high and one correction step (exact for every 32-bit p).
+struct FastDiv {
+    unsigned d, m;  // m = floor(2^32 / d), saturated for d = 1
+    __device__ __forceinline__ void divmod(unsigned p, unsigned& q, unsigned& r) const {
+        q = __umulhi(p, m);
+        r = p - q * d;
+        if (r >= d) {
+            q++;
+            r -= d;
+        }
+    }
+};
+
+inline FastDiv make_fastdiv(unsigned d) {
+    FastDiv f;
+    f.d = d;
+    f.m = d <= 1 ? 0xffffffffu : (unsigned)(0x100000000ull / d);
+    return f;
+}
+
 // DPP lane exchange inside the VALU (no LDS traffic).  `ctrl` is the DPP control word.
 template <int ctrl>
 __device__ __forceinline__ float dpp_mov(float x) {

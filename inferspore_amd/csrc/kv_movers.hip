@@ -80,25 +80,42 @@ __global__ __launch_bounds__(kBlock) void transpose_remove_padding_units(
     }
 }
 
-// cache[b, h, history[b] + t, :] = src[b, h, t, :] for t < cur_len[b]; blockIdx.z selects k / v.
-// grid = (chunks of max_q_len*seg_vec vectors, batch * kv_heads, 2), a chunk being BLOCK vectors.
-// The grid has to cover max_q_len positions per sequence (the valid lengths live on the device), so the
-// workgroups behind a sequence's end leave at once but still cost their dispatch.  Larger workgroups
-// mean fewer of them, yet measured slower (batch 8 x 32 heads, lengths 256..512 of 512: 18.5 us with
-// 256 threads, 19.0 with 512, 19.6 with 1024; the broadcast 18.5 / 19.2 / 21.8), so 256 stays the
-// default and BLOCK a tuning knob (mover_block()).
+// The grid of the two cache movers below: one workgroup per chunk of BLOCK vectors of every (sequence, head)
+// row, k / v in blockIdx.z.  The valid lengths live on the device, so the grid has to cover the maximum
+// length of every row, and the workgroups behind a sequence's end leave at once.  Which chunk a workgroup
+// takes matters more than how many leave: with chunk = blockIdx.x % chunks the live and the idle
+// workgroups repeat with the period of a row, workgroups are handed to the chip's partitions in turn, and
+// for row lengths that are multiples of the partition count (32 chunks here) some partitions then receive
+// mostly idle ones (batch 8 x 32 heads x 512 positions, every sequence 256 long: 16.1 us; lengths 256..512:
+// 18.7 us).  Rotating the chunk index by 5 per row breaks the lockstep: 12.5 and 16.9 us (copies of the same
+// bytes: 11.9 and 16.4 us); full rows are unchanged (22.5 us).  Measured and not kept: the rows as the fastest
+// grid dimension (24.9 us on full rows: neighbouring workgroups then sit 128 KiB apart), two or four
+// interleaved chunks per workgroup (23.5 / 25.1 us on full rows), workgroups of 512 and 1024 threads
+// (19.0 / 19.6 us where 256 threads take 18.5 us).
+struct MoverGrid {
+    FastDiv chunks;  // chunks per row
+    __device__ __forceinline__ void locate(unsigned& row, unsigned& chunk) const {
+        unsigned j, q, turn;
+        chunks.divmod(blockIdx.x, row, j);
+        chunks.divmod(row, q, turn);
+        chunks.divmod(j + turn * 5u, q, chunk);  // chunks <= 2^23 (a row has at most 2^31 vectors)
+    }
+};
+
+// cache[b, h, history[b] + t, :] = src[b, h, t, :] for t < cur_len[b]
 template <int BLOCK>
 __global__ __launch_bounds__(BLOCK) void concat_kv_vec(
     const char* __restrict__ k_src, const char* __restrict__ v_src, char* __restrict__ k_cache,
     char* __restrict__ v_cache, const int32_t* __restrict__ cur_query_length,
     const int32_t* __restrict__ history_length, int kv_head_num, int max_q_len, int max_seq_len,
-    SegSplit sp) {
+    SegSplit sp, MoverGrid mg) {
     const unsigned seg_vec = sp.seg_vec;
     const char* src = blockIdx.z == 0 ? k_src : v_src;
     char* cache = blockIdx.z == 0 ? k_cache : v_cache;
-    const unsigned bh = blockIdx.y;
+    unsigned bh, chunk;
+    mg.locate(bh, chunk);
     const unsigned b = bh / kv_head_num;
-    const unsigned vi = blockIdx.x * BLOCK + threadIdx.x;
+    const unsigned vi = chunk * BLOCK + threadIdx.x;
     if (vi >= (unsigned)max_q_len * seg_vec) return;
     unsigned t, c;
     sp.split(vi, t, c);
@@ -124,19 +141,19 @@ __global__ __launch_bounds__(kBlock) void concat_kv_units(
             src[((size_t)bh * max_q_len + t) * seg + i];
 }
 
-// dst[b, h, s, :] = cache[b, h / rep, s, :] for s < context_length[b]; blockIdx.z selects k / v.
-// grid = (chunks of max_k_len*seg_vec vectors, batch * heads, 2), a chunk being BLOCK vectors
+// dst[b, h, s, :] = cache[b, h / rep, s, :] for s < context_length[b]
 template <int BLOCK>
 __global__ __launch_bounds__(BLOCK) void repeat_kv_vec(
     const char* __restrict__ k_cache, const char* __restrict__ v_cache, char* __restrict__ k_dst,
     char* __restrict__ v_dst, const int32_t* __restrict__ context_length, int head_num,
-    int kv_head_num, int max_seq_len, int max_k_len, SegSplit sp) {
+    int kv_head_num, int max_seq_len, int max_k_len, SegSplit sp, MoverGrid mg) {
     const unsigned seg_vec = sp.seg_vec;
     const char* cache = blockIdx.z == 0 ? k_cache : v_cache;
     char* dst = blockIdx.z == 0 ? k_dst : v_dst;
-    const unsigned bh = blockIdx.y;
+    unsigned bh, chunk;
+    mg.locate(bh, chunk);
     const unsigned b = bh / head_num, h = bh % head_num;
-    const unsigned vi = blockIdx.x * BLOCK + threadIdx.x;
+    const unsigned vi = chunk * BLOCK + threadIdx.x;
     if (vi >= (unsigned)max_k_len * seg_vec) return;
     unsigned s, c;
     sp.split(vi, s, c);
@@ -214,7 +231,6 @@ static int concat_kv(const void* k_src, const void* v_src, void* k_cache, void* 
     ISP_REQUIRE_PTR(v_cache);
     ISP_REQUIRE_PTR(cur_query_length);
     ISP_REQUIRE_PTR(history_length);
-    if ((long long)batch * kv_head_num > kMaxGridYZ) return ISP_ERR_UNSUPPORTED;
     const size_t seg = (size_t)head_size * elem;
     // layer offset = layer * batch * kv_head_num * max_seq_len * head_size elements (concat_past_kv.cu:89)
     const size_t layer_bytes = (size_t)layer * batch * kv_head_num * max_seq_len * seg;
@@ -225,17 +241,21 @@ static int concat_kv(const void* k_src, const void* v_src, void* k_cache, void* 
     if (seg % 16 == 0 && aligned16(ks) && aligned16(vs) && aligned16(kc) && aligned16(vc)) {
         const unsigned seg_vec = (unsigned)(seg / 16);
         const size_t row_vec = (size_t)max_q_len * seg_vec;
-        if (row_vec > 0xffffffffull) return ISP_ERR_UNSUPPORTED;
+        if (row_vec > 0x7fffffffull) return ISP_ERR_UNSUPPORTED;  // 32-bit vector indices, with room for the last workgroup
         const int blk = mover_block();
-        dim3 grid((unsigned)((row_vec + blk - 1) / blk), (unsigned)(batch * kv_head_num), 2);
+        const size_t chunks = (row_vec + blk - 1) / blk;
+        if (chunks * (size_t)batch * kv_head_num > 0x7fffffffull) return ISP_ERR_UNSUPPORTED;
+        const dim3 grid((unsigned)(chunks * (size_t)batch * kv_head_num), 1, 2);
+        const MoverGrid mg{make_fastdiv((unsigned)chunks)};
 #define ISP_LAUNCH_CONCAT(B)                                                                       \
     hipLaunchKernelGGL(concat_kv_vec<B>, grid, dim3(B), 0, s, ks, vs, kc, vc, cur_query_length,     \
-                       history_length, kv_head_num, max_q_len, max_seq_len, make_split(seg_vec))
+                       history_length, kv_head_num, max_q_len, max_seq_len, make_split(seg_vec), mg)
         if (blk == 1024) ISP_LAUNCH_CONCAT(1024);
         else if (blk == 512) ISP_LAUNCH_CONCAT(512);
         else ISP_LAUNCH_CONCAT(256);
 #undef ISP_LAUNCH_CONCAT
     } else {
+        if ((long long)batch * kv_head_num > kMaxGridYZ) return ISP_ERR_UNSUPPORTED;
         const dim3 grid((unsigned)max_q_len, (unsigned)(batch * kv_head_num), 2), block(kBlock);
 #define ISP_LAUNCH_UNITS(U)                                                                        \
     hipLaunchKernelGGL(concat_kv_units<U>, grid, block, 0, s, reinterpret_cast<const U*>(ks),       \
@@ -264,7 +284,6 @@ static int repeat_kv(const void* k_cache, const void* v_cache, void* k_dst, void
     ISP_REQUIRE_PTR(k_dst);
     ISP_REQUIRE_PTR(v_dst);
     ISP_REQUIRE_PTR(context_length);
-    if ((long long)batch * head_num > kMaxGridYZ) return ISP_ERR_UNSUPPORTED;
     const size_t seg = (size_t)head_size * elem;
     const size_t layer_bytes = (size_t)layer * batch * kv_head_num * max_seq_len * seg;  // repeat_kv.cu:70
     const char* kc = static_cast<const char*>(k_cache) + layer_bytes;
@@ -274,17 +293,21 @@ static int repeat_kv(const void* k_cache, const void* v_cache, void* k_dst, void
     if (seg % 16 == 0 && aligned16(kc) && aligned16(vc) && aligned16(kd) && aligned16(vd)) {
         const unsigned seg_vec = (unsigned)(seg / 16);
         const size_t row_vec = (size_t)max_k_len * seg_vec;
-        if (row_vec > 0xffffffffull) return ISP_ERR_UNSUPPORTED;
+        if (row_vec > 0x7fffffffull) return ISP_ERR_UNSUPPORTED;  // 32-bit vector indices, with room for the last workgroup
         const int blk = mover_block();
-        dim3 grid((unsigned)((row_vec + blk - 1) / blk), (unsigned)(batch * head_num), 2);
+        const size_t chunks = (row_vec + blk - 1) / blk;
+        if (chunks * (size_t)batch * head_num > 0x7fffffffull) return ISP_ERR_UNSUPPORTED;
+        const dim3 grid((unsigned)(chunks * (size_t)batch * head_num), 1, 2);
+        const MoverGrid mg{make_fastdiv((unsigned)chunks)};
 #define ISP_LAUNCH_REPEAT(B)                                                                       \
     hipLaunchKernelGGL(repeat_kv_vec<B>, grid, dim3(B), 0, s, kc, vc, kd, vd, context_length,       \
-                       head_num, kv_head_num, max_seq_len, max_k_len, make_split(seg_vec))
+                       head_num, kv_head_num, max_seq_len, max_k_len, make_split(seg_vec), mg)
         if (blk == 1024) ISP_LAUNCH_REPEAT(1024);
         else if (blk == 512) ISP_LAUNCH_REPEAT(512);
         else ISP_LAUNCH_REPEAT(256);
 #undef ISP_LAUNCH_REPEAT
     } else {
+        if ((long long)batch * head_num > kMaxGridYZ) return ISP_ERR_UNSUPPORTED;
         const dim3 grid((unsigned)max_k_len, (unsigned)(batch * head_num), 2), block(kBlock);
 #define ISP_LAUNCH_UNITS(U)                                                                        \
     hipLaunchKernelGGL(repeat_kv_units<U>, grid, block, 0, s, reinterpret_cast<const U*>(kc),       \

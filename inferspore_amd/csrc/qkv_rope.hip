@@ -91,27 +91,6 @@ __device__ __forceinline__ void rotate_pair(float c, float sn, float x0, float x
     y1 = __fmaf_rn(c, x1, sn * x0);
 }
 
-// Unsigned division by a launch constant without the integer-divide expansion: q = floor(p / d) from
-// one multiply-high and one correction step (exact for every 32-bit p).
-struct FastDiv {
-    unsigned d, m;  // m = floor(2^32 / d), saturated for d = 1
-    __device__ __forceinline__ void divmod(unsigned p, unsigned& q, unsigned& r) const {
-        q = __umulhi(p, m);
-        r = p - q * d;
-        if (r >= d) {
-            q++;
-            r -= d;
-        }
-    }
-};
-
-static FastDiv make_fastdiv(unsigned d) {
-    FastDiv f;
-    f.d = d;
-    f.m = d <= 1 ? 0xffffffffu : (unsigned)(0x100000000ull / d);
-    return f;
-}
-
 // A wave owns kWave / G consecutive heads of one token (one head-half pair per lane: two loads and
 // two stores).  The first wave of a workgroup evaluates the token's (cos, sin) pairs (lane d
 // evaluates pair d) and shares them through LDS behind one barrier (measured 3 % faster than every

@@ -114,7 +114,8 @@ def test_argument_validation_of_the_neighbour_entry_points(lib):
     assert cat(None, None, None, None, 0, None, None, 0, 4, 8, 16, 128, None) == capi.OK
     assert cat(p, p, p, None, 0, p, p, 2, 4, 8, 16, 128, None) == capi.ERR_NULL_POINTER
     assert cat(p, p, p, p, -1, p, p, 2, 4, 8, 16, 128, None) == capi.ERR_BAD_SHAPE  # negative layer
-    assert cat(p, p, p, p, 0, p, p, 70000, 4, 8, 16, 128, None) == capi.ERR_UNSUPPORTED
+    assert cat(p, p, p, p, 0, p, p, 1 << 20, 4096, 8, 16, 128, None) == capi.ERR_UNSUPPORTED  # 2^32 workgroups
+    assert cat(p, p, p, p, 0, p, p, 70000, 4, 8, 16, 126, None) == capi.ERR_UNSUPPORTED  # row-per-workgroup form: 65535 rows
     rep = lib.isp_repeat_kv_cache_f32
     assert rep(None, None, None, None, 0, None, 0, 8, 2, 16, 8, 128, None) == capi.OK
     assert rep(p, p, p, p, 0, None, 2, 8, 2, 16, 8, 128, None) == capi.ERR_NULL_POINTER

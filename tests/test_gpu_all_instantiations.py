@@ -192,7 +192,47 @@ def test_kv_movers_every_workgroup_size(isp):
         return [t.cpu().numpy() for t in (kc, vc, kd, vd)]
 
     base = run()
+    # what the four arrays must hold, by plain indexing
+    ek = np.full((1, batch, kvn, max_seq, hs), -2.0, np.float16)
+    ev = ek.copy()
+    ekd = np.full((batch, hn, max_seq, hs), -3.0, np.float16)
+    evd = ekd.copy()
+    ks, vs = k_src.cpu().numpy(), v_src.cpu().numpy()
+    for b, (n, h0) in enumerate(zip(lens.tolist(), hist.tolist())):
+        ek[0, b, :, h0:h0 + n] = ks[b, :, :n]
+        ev[0, b, :, h0:h0 + n] = vs[b, :, :n]
+        for h in range(hn):
+            ekd[b, h, :h0 + n] = ek[0, b, h // (hn // kvn), :h0 + n]
+            evd[b, h, :h0 + n] = ev[0, b, h // (hn // kvn), :h0 + n]
+    assert all(np.array_equal(a, b) for a, b in zip(base, (ek, ev, ekd, evd)))
     for block in (256, 512, 1024):
         say("kv movers with %d-thread workgroups" % block)
         got = with_knobs({capi.TUNE_MOVER_BLOCK_THREADS: block}, run)
         assert all(np.array_equal(a, b) for a, b in zip(got, base))
+
+
+def test_kv_movers_more_rows_than_a_grid_dimension_holds(isp):
+    """A decode step of a large batch has more (sequence, head) rows than the 65535 a grid's second
+    dimension can count; the movers index their workgroups linearly, so it must simply work."""
+    batch, kvn, hn, max_seq, hs = 2100, 32, 32, 3, 128
+    say("kv movers with %d rows" % (batch * kvn))
+    g = torch.Generator(device="cuda").manual_seed(9)
+    k_src = torch.randn((batch, kvn, 1, hs), device="cuda", generator=g).half()
+    v_src = torch.randn((batch, kvn, 1, hs), device="cuda", generator=g).half()
+    lens = torch.ones(batch, dtype=torch.int32, device="cuda")
+    hist = (torch.arange(batch, device="cuda") % max_seq).to(torch.int32)
+    kc = torch.full((1, batch, kvn, max_seq, hs), -2.0, dtype=torch.float16, device="cuda")
+    vc = kc.clone()
+    isp.concat_kv_cache(k_src, v_src, 0, lens, hist, kc, vc)
+    ek = torch.full_like(kc, -2.0)
+    ev = torch.full_like(vc, -2.0)
+    rows = torch.arange(batch, device="cuda")
+    ek[0, rows, :, hist.long()] = k_src[:, :, 0]
+    ev[0, rows, :, hist.long()] = v_src[:, :, 0]
+    assert torch.equal(kc, ek) and torch.equal(vc, ev)
+    kd = torch.full((batch, hn, max_seq, hs), -3.0, dtype=torch.float16, device="cuda")
+    vd = kd.clone()
+    isp.repeat_kv_cache(kc, vc, lens + hist, 0, kd, vd)
+    live = (torch.arange(max_seq, device="cuda")[None, :] <= hist[:, None].long())[:, None, :, None]
+    assert torch.equal(kd, torch.where(live, kc[0], torch.full_like(kd, -3.0)))
+    assert torch.equal(vd, torch.where(live, vc[0], torch.full_like(vd, -3.0)))
