@@ -430,6 +430,133 @@ __global__ __launch_bounds__(512) void qkv_rope_lean_f16(
     if (APPEND && cdst != nullptr) store16_sel<ST>(cdst + cache_lane_offset, packed);
 }
 
+// The same design for 64-element heads (fp16, fully rotated, q and kv head counts multiples of 8).  A head
+// row is 128 bytes = 8 lanes; a wave carries 8 consecutive heads of one plane (q, k or v: wave-uniform), four
+// waves one token's group of 32 heads, and a workgroup of 512 threads TWO tokens, so that its first wave's
+// 64 lanes evaluate the 2 x 32 (cos, sin) pairs in one go -- per byte the same coefficient work as the
+// 128-element kernel.  Inside each row of 16 lanes the layout is [row A low | row B low | row A high |
+// row B high] (4 lanes = 64 bytes each), which puts a lane's rotation partner exactly 8 lanes away: one DPP
+// row rotation, as above, instead of two with complementary bank masks.  Every load and store instruction
+// of a wave still covers 1 KiB of whole rows.  Waves without work (odd token count, padded position, head
+// group beyond the last head) stay until the barrier and then leave.
+// `tab` MUST stay the first parameter (first_argument_word).
+template <int ST, bool BIAS, bool APPEND>
+__global__ __launch_bounds__(512) void qkv_rope_lean64_f16(
+    RopeDivisors tab, __half* q, __half* k, __half* v, const __half* qkv, const __half* bias,
+    const int32_t* __restrict__ padding_offset, const int32_t* __restrict__ history_length,
+    unsigned positions, FastDiv seq, unsigned token_num, unsigned head_num, unsigned kv_head_num,
+    KvAppend<__half> ap) {
+    constexpr unsigned ROW_BYTES = 128;
+    const unsigned tid = threadIdx.x;
+    const unsigned which = __builtin_amdgcn_readfirstlane(tid >> 8);        // first or second token
+    const unsigned w = __builtin_amdgcn_readfirstlane((tid >> 6) & 3u);     // wave inside the token
+    const unsigned token = blockIdx.x * 2u + which;
+    const unsigned qkv_heads = head_num + 2 * kv_head_num;
+    const unsigned hw = blockIdx.y * 32u + w * 8u;                          // first head of this wave
+    bool live = token < token_num && hw < qkv_heads;                        // wave-uniform
+    const unsigned l = tid & 15u;
+    const unsigned head_in_wave = ((tid & 63u) >> 4) * 2u + ((l >> 2) & 1u);
+    const unsigned g = ((l >> 3) << 2) | (l & 3u);                          // 16-byte column of the row
+    const unsigned in_block = head_in_wave * ROW_BYTES + g * 16u;
+
+    const float my_divisor = first_argument_word(tid & 31u);
+    (void)tab;
+    asm volatile("" ::: "memory");
+    // unconditional loads (a wave without work reads rows that exist and discards them): with a load
+    // inside a branch the compiler can no longer count the outstanding ones and waits for all of them
+    // where the first wave only needs its divisor
+    const unsigned token_c = token < token_num ? token : blockIdx.x * 2u;
+    const unsigned hw_c = hw < qkv_heads ? hw : 0u;
+    const vec16 raw =
+        load16_stream(reinterpret_cast<const char*>(qkv) + ((size_t)token_c * qkv_heads + hw_c) * ROW_BYTES + in_block);
+    asm volatile("" ::: "memory");
+    vec16 braw;
+    if (BIAS) braw = load16(reinterpret_cast<const char*>(bias) + (size_t)hw_c * ROW_BYTES + in_block);
+    asm volatile("" ::: "memory");
+
+    // Both tokens' positions and timesteps through scalar loads, in every wave: they run beside the vector
+    // loads above (vector memory returns in issue order, so a vector load of the padding offset would only
+    // come back behind the rows, and the first wave's evaluation with it).
+    const unsigned tok_a = blockIdx.x * 2u, tok_b = tok_a + 1u;
+    const long long p_a = (long long)tok_a + (long long)padding_offset[tok_a];
+    const long long p_b = tok_b < token_num ? (long long)tok_b + (long long)padding_offset[tok_b] : -1;
+    const bool ok_a = p_a >= 0 && p_a < (long long)positions, ok_b = p_b >= 0 && p_b < (long long)positions;
+    unsigned b_a = 0, s_a = 0, b_b = 0, s_b = 0;
+    if (ok_a) seq.divmod((unsigned)p_a, b_a, s_a);
+    if (ok_b) seq.divmod((unsigned)p_b, b_b, s_b);
+    live = live && (which ? ok_b : ok_a);
+    const unsigned b = which ? b_b : b_a, s = which ? s_b : s_a;
+
+    // Table layout [token][j][class][2]: class = the lane's column g (8 classes: 4 of the lower half row
+    // with (c, -s), 4 of the upper with (c, s)), j = 0..3 its four 16-byte reads of two (c, t) pairs each
+    __shared__ float2 cs[2][4][8][2];
+    if (blockIdx.y * 32u < head_num + kv_head_num) {  // workgroup-uniform: some wave here rotates
+        if (tid < 64) {
+            // b_a / b_b are 0 for a token without a position: both loads unconditional, so they overlap
+            const int h_a = history_length[b_a], h_b = history_length[b_b];
+            const int t_a = h_a + (int)s_a, t_b = h_b + (int)s_b;
+            const float2 coef = rope_coefficients((tid & 32u) ? t_b : t_a, my_divisor);
+            const unsigned d = tid & 31u, gg = d >> 3, e = d & 7u;  // pair d = element e of column group gg
+            cs[tid >> 5][e >> 1][gg][e & 1u] = make_float2(coef.x, -coef.y);
+            cs[tid >> 5][e >> 1][gg + 4][e & 1u] = coef;
+        }
+        __syncthreads();
+    }
+    if (!live) return;
+
+    __half* plane;
+    unsigned plane_heads, h0;
+    const bool rotates = hw < head_num + kv_head_num;
+    if (hw < head_num) {
+        plane = q, plane_heads = head_num, h0 = hw;
+    } else if (rotates) {
+        plane = k, plane_heads = kv_head_num, h0 = hw - head_num;
+    } else {
+        plane = v, plane_heads = kv_head_num, h0 = hw - head_num - kv_head_num;
+    }
+    char* dst = reinterpret_cast<char*>(plane) + (((size_t)b * plane_heads + h0) * seq.d + s) * ROW_BYTES;
+    const unsigned lane_offset = head_in_wave * (seq.d * ROW_BYTES) + g * 16u;
+    char* cdst = nullptr;
+    unsigned cache_lane_offset = 0;
+    if (APPEND && hw >= head_num) {
+        const long long row = append_row(ap, history_length, (int)b, (int)s);
+        if (row >= 0) {
+            cdst = reinterpret_cast<char*>(rotates ? ap.k_cache : ap.v_cache) +
+                   (((size_t)b * plane_heads + h0) * (size_t)ap.max_seq_len + (size_t)row) * ROW_BYTES;
+            cache_lane_offset = head_in_wave * ((unsigned)ap.max_seq_len * ROW_BYTES) + g * 16u;
+        }
+        if (plane == nullptr && cdst == nullptr) return;
+    }
+
+    if (!rotates && !BIAS) {  // v heads without bias: a plain move
+        if (!APPEND || plane != nullptr) store16_sel<ST>(dst + lane_offset, raw);
+        if (APPEND && cdst != nullptr) store16_sel<ST>(cdst + cache_lane_offset, raw);
+        return;
+    }
+    float x[8], y[8];
+    Elem<__half>::unpack(raw, x);
+    if (BIAS) {
+        float bv[8];
+        Elem<__half>::unpack(braw, bv);
+#pragma unroll
+        for (int e = 0; e < 8; e++) x[e] += bv[e];
+    }
+    if (rotates) {
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            const float2 t = cs[which][e >> 1][g][e & 1];
+            const float other = dpp_mov<0x128>(x[e]);  // row_ror:8: the other half of the same head row
+            y[e] = __fmaf_rn(t.x, x[e], t.y * other);
+        }
+    } else {
+#pragma unroll
+        for (int e = 0; e < 8; e++) y[e] = x[e];
+    }
+    const vec16 packed = Elem<__half>::pack(y);
+    if (!APPEND || plane != nullptr) store16_sel<ST>(dst + lane_offset, packed);
+    if (APPEND && cdst != nullptr) store16_sel<ST>(cdst + cache_lane_offset, packed);
+}
+
 // first_argument_word() reads the divisor table at byte 0 of the kernel's argument block, where the
 // ABI puts the first explicit parameter: fail the build if that is ever something else.
 template <typename F>
@@ -442,6 +569,9 @@ static_assert(std::is_same<FirstParameter<decltype(&qkv_rope_lean_f16<kStorePlai
                            RopeDivisors>::value &&
                   offsetof(RopeDivisors, div) == 0,
               "qkv_rope_lean_f16 must take the divisor table as its first parameter");
+static_assert(std::is_same<FirstParameter<decltype(&qkv_rope_lean64_f16<kStorePlain, false, false>)>::type,
+                           RopeDivisors>::value,
+              "qkv_rope_lean64_f16 must take the divisor table as its first parameter");
 
 // Any (even) head size and any alignment: one workgroup per token, one lane per rotation pair.
 template <typename T>
@@ -838,7 +968,38 @@ static int qkv_rope(void* q_, void* k_, void* v_, const void* qkv_, const void* 
     } else if (vec_ok && positions_ok && head_size == 128 && head_num + 2 * kv_head_num <= head_groups_max) {
         ISP_QKV_LAUNCH_WAVE(128);
         e = hipGetLastError();
-    } else if (sizeof(T) == 2 && vec_ok && positions_ok && head_size == 64 && waves_knob <= 0 &&
+    } else if (sizeof(T) == 2 && vec_ok && positions_ok && head_size == 64 && rot == 64 && waves_knob <= 0 &&
+               head_num % 8 == 0 && kv_head_num % 8 == 0 && (head_num + 2 * kv_head_num + 31) / 32 <= 65535 &&
+               (unsigned long long)seq_len * 128ull * 8ull <= 0xffffffffull &&
+               (unsigned long long)max_seq_len * 128ull * 8ull <= 0xffffffffull) {
+        // fp16 rows of 128 bytes in whole groups of 8 heads: two tokens per 512-thread workgroup
+        const dim3 g2((unsigned)((token_num + 1) / 2), (unsigned)((head_num + 2 * kv_head_num + 31) / 32));
+        __half* qh = reinterpret_cast<__half*>(q);
+        __half* kh = reinterpret_cast<__half*>(k);
+        __half* vh = reinterpret_cast<__half*>(v);
+        const __half* xh = reinterpret_cast<const __half*>(qkv);
+        const __half* bh = reinterpret_cast<const __half*>(bias);
+        KvAppend<__half> aph = {reinterpret_cast<__half*>(ap.k_cache), reinterpret_cast<__half*>(ap.v_cache),
+                                ap.input_length, ap.max_seq_len};
+        const bool with_append = aph.k_cache != nullptr;
+#define ISP_QKV_LEAN64_2(K, B, A)                                                                  \
+    hipLaunchKernelGGL((qkv_rope_lean64_f16<K, B, A>), g2, dim3(512), 0, s, tab, qh, kh, vh, xh, bh, \
+                       padding_offset, history_length, positions, fd, (unsigned)token_num,         \
+                       (unsigned)head_num, (unsigned)kv_head_num, aph)
+#define ISP_QKV_LEAN64(K)                                                                          \
+    do {                                                                                           \
+        if (bh && with_append) ISP_QKV_LEAN64_2(K, true, true);                                    \
+        else if (bh) ISP_QKV_LEAN64_2(K, true, false);                                             \
+        else if (with_append) ISP_QKV_LEAN64_2(K, false, true);                                    \
+        else ISP_QKV_LEAN64_2(K, false, false);                                                    \
+    } while (0)
+        if (kind == kStoreThrough) ISP_QKV_LEAN64(kStoreThrough);
+        else if (kind == kStoreStream) ISP_QKV_LEAN64(kStoreStream);
+        else ISP_QKV_LEAN64(kStorePlain);
+#undef ISP_QKV_LEAN64_2
+#undef ISP_QKV_LEAN64
+        e = hipGetLastError();
+    } else if (sizeof(T) == 2 && vec_ok && positions_ok && head_size == 64 && (waves_knob <= 0 || waves_knob >= 8) &&
                head_num + 2 * kv_head_num <= head_groups_max) {
         // fp16 rows of 128 bytes: one vector per lane, 8 lanes per row, 4 waves = 32 heads per workgroup
         constexpr int W = 4;

@@ -58,6 +58,7 @@ def _run_pair(isp, dtype, batch, seq, hn, kvn, hs, rot, max_seq, layers, layer, 
     (2, 9, 8, 2, 128, 128, 16),         # GQA: the general kernel
     (2, 9, 5, 1, 128, 64, 16),          # MQA, partial rotary
     (3, 7, 4, 2, 64, 64, 12),           # 64-element heads
+    (3, 7, 16, 8, 64, 64, 12),          # 64-element heads in groups of 8: two tokens per workgroup in fp16
     (2, 6, 3, 3, 16, 16, 9),            # scalar kernel
     (2, 6, 2, 1, 96, 32, 6),            # scalar kernel, partial rotary, cache too short for the longest row
 ])

@@ -317,6 +317,10 @@ def test_qkv_rope_known_answer(isp):
     (2, 6, 33, 3, 128, 128),    # head counts that are multiples of nothing
     (2, 9, 5, 1, 128, 64),      # MQA, partial rotary, head counts that do not fill a wave pass
     (3, 7, 4, 2, 64, 64),       # 64-wide heads
+    (3, 7, 32, 8, 64, 64),      # 64-wide heads in groups of 8 (fp16: two tokens per workgroup), GQA: a group of k, v and idle waves
+    (2, 9, 8, 8, 64, 64),       # same kernel, q, k and v in one group
+    (2, 5, 40, 16, 64, 64),     # same kernel, three groups, planes change inside a group
+    (2, 9, 8, 8, 64, 32),       # partial rotary keeps 64-wide heads on the whole-row kernel
     (2, 6, 3, 3, 16, 16),       # scalar kernel
     (2, 6, 2, 1, 96, 32),       # scalar kernel, partial rotary
     (1, 1, 1, 1, 2, 2),         # smallest possible

@@ -39,12 +39,15 @@ def fp16_bound(ref, positions, div):
 @pytest.mark.parametrize("store", [1, 2, 3])
 @pytest.mark.parametrize("with_bias", [False, True])
 @pytest.mark.parametrize("append", [False, True])
-def test_lean_fp16_kernel_uses_divisor_d_for_pair_d(isp, base, store, with_bias, append):
-    say("coefficients base=%g store=%d bias=%s append=%s" % (base, store, with_bias, append))
-    batch, seq, hn, hs, rot = 2, 40, 32, 128, 128
+@pytest.mark.parametrize("hs", [128, 64])
+def test_lean_fp16_kernel_uses_divisor_d_for_pair_d(isp, base, store, with_bias, append, hs):
+    say("coefficients hs=%d base=%g store=%d bias=%s append=%s" % (hs, base, store, with_bias, append))
+    # 128-element heads in groups of 32, 64-element heads in groups of 8 with an odd token count: the shapes
+    # that select the two kernels reading their divisors from the argument block
+    batch, seq, hn, rot = (2, 40, 32, 128) if hs == 128 else (2, 39, 8, 64)
     hist = np.array([0, 977], np.int32)
-    lens = np.array([seq, seq], np.int32)
-    tokens = batch * seq
+    lens = np.array([seq, seq - (hs == 64)], np.int32)
+    tokens = int(lens.sum())
     row = np.zeros(hs, np.float16)
     row[:rot // 2] = 1.0
     qkv = np.tile(row, (tokens, 3 * hn, 1))
@@ -59,6 +62,7 @@ def test_lean_fp16_kernel_uses_divisor_d_for_pair_d(isp, base, store, with_bias,
     k = torch.full_like(q, -3.0)
     v = torch.full_like(q, -3.0)
     po = torch.zeros((batch, seq), dtype=torch.int32, device="cuda")
+    po.view(-1)[lens[0]:tokens] = int(seq - lens[0])   # the second sequence starts at padded position seq
     d_hist, d_lens = torch.from_numpy(hist).cuda(), torch.from_numpy(lens).cuda()
     assert capi.lib().isp_tuning_set(capi.TUNE_QKV_STORE, store) >= 0
     try:
@@ -74,11 +78,12 @@ def test_lean_fp16_kernel_uses_divisor_d_for_pair_d(isp, base, store, with_bias,
     finally:
         capi.lib().isp_tuning_set(capi.TUNE_QKV_STORE, 0)
     for b in range(batch):
-        positions = hist[b] + np.arange(seq, dtype=np.int64)
+        n = int(lens[b])
+        positions = hist[b] + np.arange(n, dtype=np.int64)
         cos, sin, div = expected_cos_sin(positions, rot, base)
-        outs = [("q", q[b]), ("k", k[b])]
+        outs = [("q", q[b, :, :n]), ("k", k[b, :, :n])]
         if append:
-            outs.append(("k_cache", kc[0, b, :, hist[b]:hist[b] + seq, :]))
+            outs.append(("k_cache", kc[0, b, :, hist[b]:hist[b] + n, :]))
         for what, t in outs:
             got = t.cpu().numpy().astype(np.float64)                      # [heads, seq, hs]
             for half, ref in ((got[:, :, :rot // 2], cos), (got[:, :, rot // 2:], sin)):
@@ -89,7 +94,7 @@ def test_lean_fp16_kernel_uses_divisor_d_for_pair_d(isp, base, store, with_bias,
                     raise AssertionError("%s batch %d head %d position %d pair %d: got %r, closed form %r" % (
                         what, b, h, positions[s], d, half[h, s, d], ref[s, d]))
         # v is copied, not rotated
-        assert torch.equal(v[b].cpu(), torch.from_numpy(np.tile(row, (hn, seq, 1)))), "v must pass through unrotated"
+        assert torch.equal(v[b, :, :n].cpu(), torch.from_numpy(np.tile(row, (hn, n, 1)))), "v must pass through unrotated"
 
 
 def test_neighbouring_divisors_are_far_apart_in_this_test():
