@@ -96,12 +96,11 @@ __device__ __forceinline__ void rotate_pair(float c, float sn, float x0, float x
 // evaluates pair d) and shares them through LDS behind one barrier (measured 3 % faster than every
 // wave evaluating its own copy); workgroups that only carry v heads skip both.
 // grid = (tokens, head groups of WAVES waves).
-template <typename T, int HS, int ST, int WAVES>
+template <typename T, int HS, int ST, int WAVES, bool BIAS>
 __global__ __launch_bounds__(kWave * WAVES) void qkv_rope_wave(
-    T* __restrict__ q, T* __restrict__ k, T* __restrict__ v, const T* __restrict__ qkv,
-    const T* __restrict__ bias, const int32_t* __restrict__ padding_offset,
-    const int32_t* __restrict__ history_length, unsigned positions, FastDiv seq, int head_num,
-    int kv_head_num, int half_rot, RopeDivisors tab, KvAppend<T> ap) {
+    RopeDivisors tab, T* q, T* k, T* v, const T* qkv, const T* bias,
+    const int32_t* __restrict__ padding_offset, const int32_t* __restrict__ history_length,
+    unsigned positions, FastDiv seq, int head_num, int kv_head_num, int half_rot, KvAppend<T> ap) {
     constexpr int VEC = Elem<T>::kVec;
     constexpr int HALF = HS / 2;
     constexpr int G = HALF / VEC;
@@ -123,20 +122,28 @@ __global__ __launch_bounds__(kWave * WAVES) void qkv_rope_wave(
     const int h = wave_first + slot;
     const bool live = h < qkv_heads;
     const int col = g * VEC;
-    const T* src = qkv + ((size_t)token * (size_t)qkv_heads + (live ? h : 0)) * HS;
+    const int h_c = live ? h : 0;
+    const T* src = qkv + ((size_t)token * (size_t)qkv_heads + h_c) * HS;
 
     // The source address depends on the token index only, so the streamed loads are issued before
     // the destination (padding_offset -> batch row -> history) is known: the dependent scalar
-    // loads then overlap the HBM latency instead of preceding it.
-    vec16 lo, hi, blo, bhi;
-    if (live) {
-        lo = load16_stream(src + col);
-        hi = load16_stream(src + HALF + col);
-        if (bias) {
-            blo = load16(bias + (size_t)h * HS + col);
-            bhi = load16(bias + (size_t)h * HS + HALF + col);
-        }
+    // loads then overlap the HBM latency instead of preceding it.  In front of them goes the request
+    // for this lane's divisor (see first_argument_word; `tab` MUST stay the first parameter), and every
+    // load is unconditional -- lanes without a head read head 0 and discard it, the bias is a template
+    // argument -- so that the compiler can count what is outstanding and the first wave's evaluation
+    // waits for the divisor alone (with a load inside a branch it waits for everything).
+    const float my_divisor = first_argument_word((unsigned)lane);
+    (void)tab;
+    asm volatile("" ::: "memory");
+    const vec16 lo = load16_stream(src + col);
+    const vec16 hi = load16_stream(src + HALF + col);
+    asm volatile("" ::: "memory");
+    vec16 blo, bhi;
+    if (BIAS) {
+        blo = load16(bias + (size_t)h_c * HS + col);
+        bhi = load16(bias + (size_t)h_c * HS + HALF + col);
     }
+    asm volatile("" ::: "memory");
     // wave-uniform: scalar arithmetic, the division by seq_len as a multiply-high
     const long long p = (long long)token + (long long)padding_offset[token];
     if (p < 0 || p >= (long long)positions) return;
@@ -153,7 +160,7 @@ __global__ __launch_bounds__(kWave * WAVES) void qkv_rope_wave(
         __shared__ float2 cs[HALF];
         if (wave == 0 && lane < HALF) {
             float2 coef = make_float2(1.0f, 0.0f);
-            if (lane < half_rot) coef = rope_coefficients(history_length[b] + s, tab.div[lane]);
+            if (lane < half_rot) coef = rope_coefficients(history_length[b] + s, my_divisor);
             cs[lane] = coef;
         }
         __syncthreads();
@@ -169,7 +176,7 @@ __global__ __launch_bounds__(kWave * WAVES) void qkv_rope_wave(
     float x0[VEC], x1[VEC];
     Elem<T>::unpack(lo, x0);
     Elem<T>::unpack(hi, x1);
-    if (bias) {
+    if (BIAS) {
         float b0[VEC], b1[VEC];
         Elem<T>::unpack(blo, b0);
         Elem<T>::unpack(bhi, b1);
@@ -572,6 +579,9 @@ static_assert(std::is_same<FirstParameter<decltype(&qkv_rope_lean_f16<kStorePlai
 static_assert(std::is_same<FirstParameter<decltype(&qkv_rope_lean64_f16<kStorePlain, false, false>)>::type,
                            RopeDivisors>::value,
               "qkv_rope_lean64_f16 must take the divisor table as its first parameter");
+static_assert(std::is_same<FirstParameter<decltype(&qkv_rope_wave<float, 128, kStorePlain, 4, false>)>::type,
+                           RopeDivisors>::value,
+              "qkv_rope_wave must take the divisor table as its first parameter");
 
 // Any (even) head size and any alignment: one workgroup per token, one lane per rotation pair.
 template <typename T>
@@ -908,9 +918,14 @@ static int qkv_rope(void* q_, void* k_, void* v_, const void* qkv_, const void* 
     do {                                                                                           \
         constexpr int HPB = (kWave / ((HS / 2) / Elem<T>::kVec)) * W;                              \
         dim3 g2((unsigned)token_num, (unsigned)((head_num + 2 * kv_head_num + HPB - 1) / HPB));    \
-        hipLaunchKernelGGL((qkv_rope_wave<T, HS, K, W>), g2, dim3(kWave * W), 0, s, q, k, v, qkv,   \
-                           bias, padding_offset, history_length, positions, fd, head_num,          \
-                           kv_head_num, half_rot, tab, ap);                                        \
+        if (bias)                                                                                  \
+            hipLaunchKernelGGL((qkv_rope_wave<T, HS, K, W, true>), g2, dim3(kWave * W), 0, s, tab, q,  \
+                               k, v, qkv, bias, padding_offset, history_length, positions, fd,     \
+                               head_num, kv_head_num, half_rot, ap);                               \
+        else                                                                                       \
+            hipLaunchKernelGGL((qkv_rope_wave<T, HS, K, W, false>), g2, dim3(kWave * W), 0, s, tab, q, \
+                               k, v, qkv, bias, padding_offset, history_length, positions, fd,     \
+                               head_num, kv_head_num, half_rot, ap);                               \
     } while (0)
 #define ISP_QKV_LAUNCH_K(HS, W)                                                                    \
     do {                                                                                           \
