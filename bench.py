@@ -220,7 +220,7 @@ def make_workloads(torch, lib, stream_handle, rotate):
         if es == 2 and hs == 128 and hn % 32 == 0 and kvn % 32 == 0:
             w.kernel = "isp::qkv_rope_lean_f16<2, true, false>"
         else:
-            w.kernel = "isp::qkv_rope_wave<%s, %d, 2, 4>" % ("__half" if es == 2 else "float", hs)
+            w.kernel = "isp::qkv_rope_wave<%s, %d, 2, 4, true>" % ("__half" if es == 2 else "float", hs)
         w.bytes_per_launch = tokens * (2 * (hn + 2 * kvn) * hs * es + 4) + (hn + 2 * kvn) * hs * es + 2 * batch * 4
         hist = torch.zeros(batch, device=dev, dtype=torch.int32)
         bias = (0.02 * torch.randn((hn + 2 * kvn) * hs, device=dev)).to(tdtype)
