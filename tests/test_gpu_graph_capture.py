@@ -145,3 +145,72 @@ def test_capture_of_the_prefill_kernels(isp):
         isp.add_fused_qkv_bias_transpose_and_rope(other, other.clone(), other.clone(), t["qkv"], None, t["po"],
                                                   t["hist"], lens, 128, 500000.0)
         torch.cuda.synchronize()
+
+
+def test_capture_of_the_fused_entry_points(isp):
+    """The fused forms under capture: the prefill step with the KV append (fp16 with 64-element heads, whose
+    kernel reads its divisors out of the argument block, and fp32 through the general kernel, which does the
+    same) and the decode step (bias + RoPE + append in one launch).  Each replay continues where the last one
+    stopped: the decode step rotates its buffer in place, so three replays must equal three eager steps."""
+    print("[case] graph capture of the fused entry points", flush=True)
+    g = torch.Generator(device="cuda").manual_seed(5)
+    batch, seq, max_seq = 3, 20, 64
+    lens = torch.tensor([20, 7, 13], dtype=torch.int32, device="cuda")
+    tokens = int(lens.sum())
+    hist = torch.tensor([0, 30, 5], dtype=torch.int32, device="cuda")
+    t = {"po": torch.zeros((batch, seq), dtype=torch.int32, device="cuda"),
+         "cum": torch.zeros((batch + 1,), dtype=torch.int32, device="cuda")}
+    shapes = {"h": (torch.float16, 16, 8, 64), "f": (torch.float32, 8, 2, 128)}
+    for tag, (dt, hn, kvn, hs) in shapes.items():
+        r = lambda *s: torch.randn(s, device="cuda", generator=g).to(dt)
+        t.update({
+            tag + "qkv": r(tokens, hn + 2 * kvn, hs), tag + "bias": r((hn + 2 * kvn) * hs) * 0.1,
+            tag + "q": torch.zeros((batch, hn, seq, hs), dtype=dt, device="cuda"),
+            tag + "kc": torch.zeros((2, batch, kvn, max_seq, hs), dtype=dt, device="cuda"),
+            tag + "vc": torch.zeros((2, batch, kvn, max_seq, hs), dtype=dt, device="cuda"),
+            tag + "step_qkv": r(batch, hn + 2 * kvn, hs),
+        })
+
+    ctx = hist + lens          # allocated before the capture: the sequence itself must not allocate
+
+    def sequence():
+        isp.cal_padding_offset(t["po"], t["cum"], lens)
+        for tag, (dt, hn, kvn, hs) in shapes.items():
+            isp.add_fused_qkv_bias_transpose_rope_and_append(t[tag + "q"], None, None, t[tag + "kc"], t[tag + "vc"], 1,
+                                                             t[tag + "qkv"], t[tag + "bias"], t["po"], hist, lens, hs,
+                                                             10000.0)
+            isp.rope_decode_and_append(t[tag + "step_qkv"], t[tag + "bias"], t[tag + "kc"], t[tag + "vc"], 0, ctx,
+                                       41, hn, hs, 10000.0)
+
+    initial = _snapshot(t)
+    eager = []
+    for _ in range(3):
+        sequence()
+        torch.cuda.synchronize()
+        eager.append(_snapshot(t))
+    assert not torch.equal(eager[0]["hstep_qkv"], eager[1]["hstep_qkv"]), "the decode step must work in place"
+    for k, v in initial.items():
+        t[k].copy_(v)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        sequence()
+        for k, v in initial.items():
+            t[k].copy_(v)
+        side.synchronize()
+        graph.capture_begin()
+        sequence()
+        graph.capture_end()
+    torch.cuda.synchronize()
+    for step in range(3):
+        graph.replay()
+        torch.cuda.synchronize()
+        for k, v in eager[step].items():
+            assert torch.equal(t[k], v), "replay %d differs from eager in %s" % (step, k)
+        # the same kernels with other arguments between the replays
+        other = torch.zeros_like(t["hq"])
+        isp.add_fused_qkv_bias_transpose_rope_and_append(other, None, None, torch.zeros_like(t["hkc"]),
+                                                         torch.zeros_like(t["hvc"]), 0, t["hqkv"], None, t["po"], hist,
+                                                         lens, 64, 500000.0)
+        torch.cuda.synchronize()
