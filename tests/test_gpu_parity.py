@@ -151,8 +151,6 @@ def test_fused_norm_known_answer(isp):
 @pytest.mark.parametrize("tokens,hidden", [(2048, 4096), (7, 4096), (1, 8), (13, 1000), (5, 8192), (3, 11008),
                                            (2, 16384), (9, 520)])
 def test_fused_norm_variants(isp, oracle, dtype, wpr, tokens, hidden):
-    if tokens == 2048 and dtype == np.float32 and wpr not in (0, 4):
-        pytest.skip("covered by the fp16 sweep")
     say("fused norm %s %dx%d wpr=%d" % (dtype.__name__, tokens, hidden, wpr))
     _check_norm(isp, oracle, dtype, tokens, hidden, True, True, wpr=wpr, seed=tokens + hidden)
 
