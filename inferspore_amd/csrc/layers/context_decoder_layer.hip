@@ -7,6 +7,8 @@
 #include <hipblaslt/hipblaslt.h>
 
 #include <cmath>
+#include <cstdlib>
+#include <cstring>
 #include <map>
 #include <string>
 #include <tuple>
@@ -44,9 +46,16 @@ struct LtType<half> {
 //             q x k^T), else [k, n].
 // hipBLASLt is column-major, so the call computes C^T = op(W)^T x A^T: its "A" operand is W, its
 // "B" operand is the activation, and a row-major [r, c] matrix is a column-major [c, r] one.
+//
+// The algorithm of a shape is chosen once, when the shape is first seen: the library's heuristic proposes
+// up to kCandidates, and unless ISP_LAYERS_GEMM_AUTOTUNE=0 each is run on the call's own operands (beta is
+// 0 and no output aliases an input, so repeating the product is harmless) and the fastest is kept -- the
+// first proposal is not always the fastest on a given device.
 class GemmEngine {
 public:
     explicit GemmEngine(BaseAllocator* allocator) : allocator_(allocator) {
+        const char* env = std::getenv("ISP_LAYERS_GEMM_AUTOTUNE");
+        autotune_ = !(env != nullptr && std::strcmp(env, "0") == 0);
         ISP_LT_CHECK(hipblasLtCreate(&handle_));
         workspace_ = allocator_->UnifyMalloc(nullptr, kWorkspaceBytes, false);
         ISP_LT_CHECK(hipblasLtMatmulPreferenceCreate(&pref_));
@@ -69,7 +78,7 @@ public:
         if (m == 0 || n == 0 || batch == 0) return;
         const Key key{(int)type, m, n, k, w_is_nk ? 1 : 0, lda, ldw, ldc, batch, stride_a, stride_w, stride_c};
         auto it = plans_.find(key);
-        if (it == plans_.end()) it = plans_.emplace(key, plan(type, key)).first;
+        if (it == plans_.end()) it = plans_.emplace(key, plan(type, key, a, w, c, alpha)).first;
         const Plan& p = it->second;
         const float beta = 0.0f;
         ISP_LT_CHECK(hipblasLtMatmul(handle_, p.desc, &alpha, w, p.w, a, p.a, &beta, c, p.c, c, p.c, &p.algo,
@@ -78,6 +87,7 @@ public:
 
 private:
     static constexpr size_t kWorkspaceBytes = 32u << 20;
+    static constexpr int kCandidates = 8;
     using Key = std::tuple<int, int, int, int, int, int, int, int, int, long long, long long, long long>;
     struct Plan {
         hipblasLtMatmulDesc_t desc = nullptr;
@@ -94,7 +104,35 @@ private:
                                                        sizeof(offset)));
     }
 
-    Plan plan(hipDataType type, const Key& key) {
+    // Milliseconds per product with `algo` (two untimed runs, then the mean of five); negative if it fails.
+    float time_algo(const Plan& p, const hipblasLtMatmulAlgo_t& algo, const void* a, const void* w, void* c,
+                    float alpha) {
+        const float beta = 0.0f;
+        hipEvent_t e0, e1;
+        if (hipEventCreate(&e0) != hipSuccess) return -1.0f;
+        if (hipEventCreate(&e1) != hipSuccess) {
+            (void)hipEventDestroy(e0);
+            return -1.0f;
+        }
+        float ms = -1.0f;
+        bool ok = true;
+        for (int i = 0; i < 7 && ok; i++) {
+            if (i == 2) ok = hipEventRecord(e0, nullptr) == hipSuccess;
+            ok = ok && hipblasLtMatmul(handle_, p.desc, &alpha, w, p.w, a, p.a, &beta, c, p.c, c, p.c, &algo,
+                                       workspace_, kWorkspaceBytes, nullptr) == HIPBLAS_STATUS_SUCCESS;
+        }
+        if (ok && hipEventRecord(e1, nullptr) == hipSuccess && hipEventSynchronize(e1) == hipSuccess &&
+            hipEventElapsedTime(&ms, e0, e1) == hipSuccess)
+            ms /= 5.0f;
+        else
+            ms = -1.0f;
+        (void)hipGetLastError();
+        (void)hipEventDestroy(e0);
+        (void)hipEventDestroy(e1);
+        return ms;
+    }
+
+    Plan plan(hipDataType type, const Key& key, const void* a, const void* w, void* c, float alpha) {
         int m, n, k, nk, lda, ldw, ldc, batch, t;
         long long sa, sw, sc;
         std::tie(t, m, n, k, nk, lda, ldw, ldc, batch, sa, sw, sc) = key;
@@ -112,11 +150,24 @@ private:
         batched(p.w, batch, sw);
         batched(p.a, batch, sa);
         batched(p.c, batch, sc);
-        hipblasLtMatmulHeuristicResult_t found[1];
+        hipblasLtMatmulHeuristicResult_t found[kCandidates];
         int count = 0;
-        ISP_LT_CHECK(hipblasLtMatmulAlgoGetHeuristic(handle_, p.desc, p.w, p.a, p.c, p.c, pref_, 1, found, &count));
+        ISP_LT_CHECK(hipblasLtMatmulAlgoGetHeuristic(handle_, p.desc, p.w, p.a, p.c, p.c, pref_,
+                                                     autotune_ ? kCandidates : 1, found, &count));
         LLM_CHECK_WITH_INFO(count > 0, "hipBLASLt offers no algorithm for a GEMM of this layer");
-        p.algo = found[0].algo;
+        int best = 0;
+        if (autotune_ && count > 1) {
+            float best_ms = -1.0f;
+            for (int i = 0; i < count; i++) {
+                if (found[i].workspaceSize > kWorkspaceBytes) continue;
+                const float ms = time_algo(p, found[i].algo, a, w, c, alpha);
+                if (ms >= 0.0f && (best_ms < 0.0f || ms < best_ms)) {
+                    best_ms = ms;
+                    best = i;
+                }
+            }
+        }
+        p.algo = found[best].algo;
         return p;
     }
 
@@ -131,6 +182,7 @@ private:
     hipblasLtHandle_t handle_ = nullptr;
     hipblasLtMatmulPreference_t pref_ = nullptr;
     void* workspace_ = nullptr;
+    bool autotune_ = true;
     std::map<Key, Plan> plans_;
 };
 
@@ -184,6 +236,99 @@ __global__ __launch_bounds__(256) void masked_scaled_softmax(T* scores, const in
         const float p = i < visible ? expf(scale * to_float(row[i]) - m) * inv : 0.0f;
         from_float(p, row + i);
     }
+}
+
+// The same, one wavefront per row with the row in registers: NVW 16-byte vectors per lane cover rows of
+// up to 64 * NVW vectors (512 * NVW fp16 keys), every element is read once and written once, vectors that
+// lie wholly behind the visible keys are not read at all, and rows of padded queries are only zeroed.
+// exp through the hardware exponential (relative error about 2^-22, far inside what the attention
+// output is compared at).  Used when max_k_len is a whole number of vectors and fits; else the kernel above.
+template <typename T, int NVW>
+__global__ __launch_bounds__(256) void masked_scaled_softmax_rows(T* scores, const int* history_length,
+                                                                  const int* input_length,
+                                                                  const int* context_length, int head_num,
+                                                                  int max_q_len, int max_k_len, float scale,
+                                                                  long long rows) {
+    constexpr int VEC = 16 / (int)sizeof(T);
+    union Vec16 {
+        uint4 raw;
+        T e[VEC];
+    };
+    const int lane = threadIdx.x % 64;
+    const long long row_id = (long long)blockIdx.x * 4 + threadIdx.x / 64;
+    if (row_id >= rows) return;  // wave-uniform
+    const int q = (int)(row_id % max_q_len);
+    const int b = (int)(row_id / max_q_len / head_num);
+    int visible = 0;
+    if (q < input_length[b]) {
+        visible = history_length[b] + q + 1;
+        if (visible > context_length[b]) visible = context_length[b];
+        if (visible > max_k_len) visible = max_k_len;
+    }
+    T* row = scores + (size_t)row_id * (size_t)max_k_len;
+    const int nvec = max_k_len / VEC;
+    float x[NVW][VEC];
+    float m = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < NVW; j++) {
+        const int vi = lane + 64 * j, k0 = vi * VEC;
+        Vec16 v;
+        const bool have = vi < nvec && k0 < visible;
+        if (have) v.raw = *reinterpret_cast<const uint4*>(row + k0);
+#pragma unroll
+        for (int e = 0; e < VEC; e++) {
+            x[j][e] = (have && k0 + e < visible) ? scale * to_float(v.e[e]) : -INFINITY;
+            m = fmaxf(m, x[j][e]);
+        }
+    }
+    for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off, 64));
+    float sum = 0.0f;
+#pragma unroll
+    for (int j = 0; j < NVW; j++) {
+#pragma unroll
+        for (int e = 0; e < VEC; e++) {
+            x[j][e] = x[j][e] == -INFINITY ? 0.0f : __expf(x[j][e] - m);
+            sum += x[j][e];
+        }
+    }
+    for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
+    const float inv = visible > 0 ? 1.0f / sum : 0.0f;
+#pragma unroll
+    for (int j = 0; j < NVW; j++) {
+        const int vi = lane + 64 * j;
+        if (vi < nvec) {
+            Vec16 v;
+#pragma unroll
+            for (int e = 0; e < VEC; e++) from_float(x[j][e] * inv, &v.e[e]);
+            *reinterpret_cast<uint4*>(row + vi * VEC) = v.raw;
+        }
+    }
+}
+
+template <typename T>
+void launch_masked_scaled_softmax(T* scores, const int* history_length, const int* input_length,
+                                  const int* context_length, int batch, int head_num, int max_q_len,
+                                  int max_k_len, float scale) {
+    constexpr int VEC = 16 / (int)sizeof(T);
+    const long long rows = (long long)batch * head_num * max_q_len;
+    const int nvec = max_k_len / VEC;
+    const bool rows_ok = max_k_len % VEC == 0 && nvec <= 64 * 4 && (reinterpret_cast<uintptr_t>(scores) & 15u) == 0 &&
+                         (rows + 3) / 4 <= 0x7fffffffLL;
+    if (rows_ok) {
+        const dim3 grid((unsigned)((rows + 3) / 4)), block(256);
+#define ISP_SOFTMAX_ROWS(N)                                                                              \
+    hipLaunchKernelGGL((masked_scaled_softmax_rows<T, N>), grid, block, 0, nullptr, scores, history_length, \
+                       input_length, context_length, head_num, max_q_len, max_k_len, scale, rows)
+        if (nvec <= 64) ISP_SOFTMAX_ROWS(1);
+        else if (nvec <= 128) ISP_SOFTMAX_ROWS(2);
+        else ISP_SOFTMAX_ROWS(4);
+#undef ISP_SOFTMAX_ROWS
+    } else {
+        hipLaunchKernelGGL((masked_scaled_softmax<T>), dim3((unsigned)max_q_len, (unsigned)head_num, (unsigned)batch),
+                           dim3(256), 0, nullptr, scores, history_length, input_length, context_length, head_num,
+                           max_q_len, max_k_len, scale);
+    }
+    CHECK(hipGetLastError());
 }
 
 }  // namespace isp_layers
@@ -334,10 +479,8 @@ void LlamaContextDecoderLayer<T>::forward(TensorMap& inputs, LlamaLayerWeight<T>
     const int bh = batch * head_num_;
     gemm_->matmul(lt, q_buf_, k_all_, scores_, max_q, max_k, hs, true, hs, hs, max_k, bh, (long long)max_q * hs,
                   (long long)max_k * hs, (long long)max_q * max_k);
-    hipLaunchKernelGGL((isp_layers::masked_scaled_softmax<T>), dim3((unsigned)max_q, (unsigned)head_num_, (unsigned)batch),
-                       dim3(256), 0, nullptr, scores_, history_length->data, input_length->data, context_length->data,
-                       head_num_, max_q, max_k, 1.0f / std::sqrt((float)hs));
-    CHECK(hipGetLastError());
+    isp_layers::launch_masked_scaled_softmax(scores_, history_length->data, input_length->data, context_length->data,
+                                             batch, head_num_, max_q, max_k, 1.0f / std::sqrt((float)hs));
     gemm_->matmul(lt, scores_, v_all_, ctx_, max_q, hs, max_k, false, max_k, hs, hs, bh, (long long)max_q * max_k,
                   (long long)max_k * hs, (long long)max_q * hs);
     // 5. [batch, heads, max_q, hs] -> packed [tokens, heads, hs]
