@@ -3,6 +3,7 @@
 
 #include <hip/hip_fp16.h>
 #include <hip/hip_runtime.h>
+
 #include <stdint.h>
 
 #include "inferspore_amd.h"
@@ -241,6 +242,17 @@ inline FastDiv make_fastdiv(unsigned d) {
     f.d = d;
     f.m = d <= 1 ? 0xffffffffu : (unsigned)(0x100000000ull / d);
     return f;
+}
+
+// p[i] of an int32 array that no kernel of this library writes (token ids, sequence lengths), read through
+// the constant address space so that a wave-uniform index takes the scalar path.  A __restrict__ kernel
+// parameter gets that by itself; a pointer inside an argument struct, or one that has been named in an
+// asm statement, does not: the compiler must then assume that the kernel's own stores could alias it,
+// issues a vector load and waits for every earlier vector load -- the streamed rows -- before it looks at
+// the value (fused KV append: 26.8 -> 26.05 us).
+__device__ __forceinline__ int32_t read_only_i32(const int32_t* p, int i) {
+    typedef const int32_t __attribute__((address_space(4)))* constant_ints;
+    return reinterpret_cast<constant_ints>((unsigned long long)p)[i];
 }
 
 // DPP lane exchange inside the VALU (no LDS traffic).  `ctrl` is the DPP control word.

@@ -48,15 +48,18 @@ static SegSplit make_split(unsigned seg_vec) {
 // grid = tokens * chunks, a chunk being 256 vectors of the token's heads*seg_vec vectors
 __global__ __launch_bounds__(kBlock) void transpose_remove_padding_vec(
     const char* __restrict__ src, const int32_t* __restrict__ padding_offset, char* __restrict__ dst,
-    int batch, int head_num, int seq_len, SegSplit sp, unsigned chunks) {
+    unsigned positions, int head_num, FastDiv seq, SegSplit sp, FastDiv chunks) {
     const unsigned seg_vec = sp.seg_vec;
-    const unsigned token = blockIdx.x / chunks;
-    const unsigned vi = (blockIdx.x % chunks) * kBlock + threadIdx.x;  // vector index inside the token's row
+    const unsigned seq_len = seq.d;
+    unsigned token, chunk;
+    chunks.divmod(blockIdx.x, token, chunk);
+    const unsigned vi = chunk * kBlock + threadIdx.x;  // vector index inside the token's row
     const unsigned row_vec = (unsigned)head_num * seg_vec;
     if (vi >= row_vec) return;
-    const long long p = (long long)token + (long long)padding_offset[token];
-    if (p < 0 || p >= (long long)batch * seq_len) return;
-    const unsigned b = (unsigned)(p / seq_len), s = (unsigned)(p % seq_len);
+    const long long p = (long long)token + (long long)read_only_i32(padding_offset, (int)token);
+    if (p < 0 || p >= (long long)positions) return;
+    unsigned b, s;
+    seq.divmod((unsigned)p, b, s);
     unsigned h, c;
     sp.split(vi, h, c);
     const size_t from = ((((size_t)b * head_num + h) * seq_len + s) * seg_vec + c) * 16u;
@@ -107,20 +110,21 @@ template <int BLOCK>
 __global__ __launch_bounds__(BLOCK) void concat_kv_vec(
     const char* __restrict__ k_src, const char* __restrict__ v_src, char* __restrict__ k_cache,
     char* __restrict__ v_cache, const int32_t* __restrict__ cur_query_length,
-    const int32_t* __restrict__ history_length, int kv_head_num, int max_q_len, int max_seq_len,
+    const int32_t* __restrict__ history_length, FastDiv kv_heads, int max_q_len, int max_seq_len,
     SegSplit sp, MoverGrid mg) {
     const unsigned seg_vec = sp.seg_vec;
     const char* src = blockIdx.z == 0 ? k_src : v_src;
     char* cache = blockIdx.z == 0 ? k_cache : v_cache;
     unsigned bh, chunk;
     mg.locate(bh, chunk);
-    const unsigned b = bh / kv_head_num;
+    unsigned b, head;
+    kv_heads.divmod(bh, b, head);
     const unsigned vi = chunk * BLOCK + threadIdx.x;
     if (vi >= (unsigned)max_q_len * seg_vec) return;
     unsigned t, c;
     sp.split(vi, t, c);
-    const int cur = cur_query_length[b];
-    const long long row = (long long)history_length[b] + t;
+    const int cur = read_only_i32(cur_query_length, (int)b);
+    const long long row = (long long)read_only_i32(history_length, (int)b) + t;
     if ((int)t >= cur || row < 0 || row >= max_seq_len) return;
     store16_through(cache + (((size_t)bh * max_seq_len + (size_t)row) * seg_vec + c) * 16u,
                    load16_stream(src + ((size_t)bh * max_q_len * seg_vec + vi) * 16u));
@@ -145,20 +149,22 @@ __global__ __launch_bounds__(kBlock) void concat_kv_units(
 template <int BLOCK>
 __global__ __launch_bounds__(BLOCK) void repeat_kv_vec(
     const char* __restrict__ k_cache, const char* __restrict__ v_cache, char* __restrict__ k_dst,
-    char* __restrict__ v_dst, const int32_t* __restrict__ context_length, int head_num,
+    char* __restrict__ v_dst, const int32_t* __restrict__ context_length, FastDiv heads, FastDiv group,
     int kv_head_num, int max_seq_len, int max_k_len, SegSplit sp, MoverGrid mg) {
     const unsigned seg_vec = sp.seg_vec;
     const char* cache = blockIdx.z == 0 ? k_cache : v_cache;
     char* dst = blockIdx.z == 0 ? k_dst : v_dst;
     unsigned bh, chunk;
     mg.locate(bh, chunk);
-    const unsigned b = bh / head_num, h = bh % head_num;
+    unsigned b, h;
+    heads.divmod(bh, b, h);
     const unsigned vi = chunk * BLOCK + threadIdx.x;
     if (vi >= (unsigned)max_k_len * seg_vec) return;
     unsigned s, c;
     sp.split(vi, s, c);
-    if ((int)s >= context_length[b] || (int)s >= max_seq_len) return;
-    const unsigned kvh = h / (unsigned)(head_num / kv_head_num);
+    if ((int)s >= read_only_i32(context_length, (int)b) || (int)s >= max_seq_len) return;
+    unsigned kvh, within;
+    group.divmod(h, kvh, within);
     store16_through(dst + ((size_t)bh * max_k_len * seg_vec + vi) * 16u,
                    load16_stream(cache + (((size_t)b * kv_head_num + kvh) * max_seq_len * seg_vec + vi) * 16u));
 }
@@ -197,12 +203,15 @@ static int transpose_remove_padding(const void* src, const int32_t* padding_offs
     ISP_REQUIRE_PTR(dst);
     const size_t seg = (size_t)head_size * elem;
     const size_t chunks = ((size_t)head_num * (seg / 16) + kBlock - 1) / kBlock;
-    if (seg % 16 == 0 && aligned16(src) && aligned16(dst) && chunks * (size_t)token_num <= 0x7fffffffull) {
+    // the vector kernel keeps padded positions in 32 bits and divides with a multiply-high
+    if (seg % 16 == 0 && aligned16(src) && aligned16(dst) && chunks * (size_t)token_num <= 0x7fffffffull &&
+        (unsigned long long)batch * (unsigned long long)seq_len <= 0x7fffffffull) {
         const unsigned seg_vec = (unsigned)(seg / 16);
         dim3 grid((unsigned)(chunks * (size_t)token_num));
         hipLaunchKernelGGL(transpose_remove_padding_vec, grid, dim3(kBlock), 0, s,
                            static_cast<const char*>(src), padding_offset, static_cast<char*>(dst),
-                           batch, head_num, seq_len, make_split(seg_vec), (unsigned)chunks);
+                           (unsigned)batch * (unsigned)seq_len, head_num, make_fastdiv((unsigned)seq_len),
+                           make_split(seg_vec), make_fastdiv((unsigned)chunks));
     } else {
         const dim3 grid((unsigned)token_num), block(kBlock);
 #define ISP_LAUNCH_UNITS(U)                                                                        \
@@ -249,7 +258,8 @@ static int concat_kv(const void* k_src, const void* v_src, void* k_cache, void* 
         const MoverGrid mg{make_fastdiv((unsigned)chunks)};
 #define ISP_LAUNCH_CONCAT(B)                                                                       \
     hipLaunchKernelGGL(concat_kv_vec<B>, grid, dim3(B), 0, s, ks, vs, kc, vc, cur_query_length,     \
-                       history_length, kv_head_num, max_q_len, max_seq_len, make_split(seg_vec), mg)
+                       history_length, make_fastdiv((unsigned)kv_head_num), max_q_len, max_seq_len,       \
+                       make_split(seg_vec), mg)
         if (blk == 1024) ISP_LAUNCH_CONCAT(1024);
         else if (blk == 512) ISP_LAUNCH_CONCAT(512);
         else ISP_LAUNCH_CONCAT(256);
@@ -301,7 +311,8 @@ static int repeat_kv(const void* k_cache, const void* v_cache, void* k_dst, void
         const MoverGrid mg{make_fastdiv((unsigned)chunks)};
 #define ISP_LAUNCH_REPEAT(B)                                                                       \
     hipLaunchKernelGGL(repeat_kv_vec<B>, grid, dim3(B), 0, s, kc, vc, kd, vd, context_length,       \
-                       head_num, kv_head_num, max_seq_len, max_k_len, make_split(seg_vec), mg)
+                       make_fastdiv((unsigned)head_num), make_fastdiv((unsigned)(head_num / kv_head_num)),    \
+                       kv_head_num, max_seq_len, max_k_len, make_split(seg_vec), mg)
         if (blk == 1024) ISP_LAUNCH_REPEAT(1024);
         else if (blk == 512) ISP_LAUNCH_REPEAT(512);
         else ISP_LAUNCH_REPEAT(256);

@@ -52,20 +52,10 @@ struct KvAppend {
 };
 
 // Row of the cache a token at (b, s) is appended to, or -1.
-// p[i] for a pointer that arrives inside an argument struct (where __restrict__ means nothing) and whose
-// target no kernel of this file writes: read through the constant address space, so that a wave-uniform
-// index takes the scalar path.  As an ordinary global pointer the compiler must assume that the kernel's
-// own stores could alias it, issues a vector load and then waits for every earlier vector load -- the
-// streamed rows -- before it looks at the value (fused append: 26.7 -> 26.0 us).
-__device__ __forceinline__ int32_t read_only_i32(const int32_t* p, int i) {
-    typedef const int32_t __attribute__((address_space(4)))* constant_ints;
-    return reinterpret_cast<constant_ints>((unsigned long long)p)[i];
-}
-
 template <typename T>
 __device__ __forceinline__ long long append_row(const KvAppend<T>& ap, const int32_t* history_length, int b, int s) {
     if (ap.k_cache == nullptr || s >= read_only_i32(ap.input_length, b)) return -1;
-    const long long row = (long long)history_length[b] + s;
+    const long long row = (long long)read_only_i32(history_length, b) + s;
     return (row >= 0 && row < ap.max_seq_len) ? row : -1;
 }
 
@@ -155,7 +145,7 @@ __global__ __launch_bounds__(kWave * WAVES) void qkv_rope_wave(
     }
     asm volatile("" ::: "memory");
     // wave-uniform: scalar arithmetic, the division by seq_len as a multiply-high
-    const long long p = (long long)token + (long long)padding_offset[token];
+    const long long p = (long long)token + (long long)read_only_i32(padding_offset, (int)token);
     if (p < 0 || p >= (long long)positions) return;
     unsigned ub, us;
     seq.divmod((unsigned)p, ub, us);
@@ -170,7 +160,7 @@ __global__ __launch_bounds__(kWave * WAVES) void qkv_rope_wave(
         __shared__ float2 cs[HALF];
         if (wave == 0 && lane < HALF) {
             float2 coef = make_float2(1.0f, 0.0f);
-            if (lane < half_rot) coef = rope_coefficients(history_length[b] + s, my_divisor);
+            if (lane < half_rot) coef = rope_coefficients(read_only_i32(history_length, b) + s, my_divisor);
             cs[lane] = coef;
         }
         __syncthreads();
@@ -264,7 +254,7 @@ __global__ __launch_bounds__(kWave * WAVES) void qkv_rope_rows64_f16(
         raw = load16_stream(qkv + ((size_t)token * (size_t)qkv_heads + h) * HS + col);
         if (bias) braw = load16(bias + (size_t)h * HS + col);
     }
-    const long long p = (long long)token + (long long)padding_offset[token];
+    const long long p = (long long)token + (long long)read_only_i32(padding_offset, (int)token);
     if (p < 0 || p >= (long long)positions) return;  // workgroup-uniform
     unsigned ub, us;
     seq.divmod((unsigned)p, ub, us);
@@ -279,7 +269,7 @@ __global__ __launch_bounds__(kWave * WAVES) void qkv_rope_rows64_f16(
         __shared__ float2 cs[HALF];
         if (wave == 0 && lane < HALF) {
             float2 coef = make_float2(1.0f, 0.0f);
-            if (lane < half_rot) coef = rope_coefficients(history_length[b] + s, tab.div[lane]);
+            if (lane < half_rot) coef = rope_coefficients(read_only_i32(history_length, b) + s, tab.div[lane]);
             cs[lane] = coef;
         }
         __syncthreads();
@@ -373,7 +363,7 @@ __global__ __launch_bounds__(512) void qkv_rope_lean_f16(
     if (BIAS) braw = load16(reinterpret_cast<const char*>(bias) + (size_t)first * ROW_BYTES + tid * 16u);
     asm volatile("" ::: "memory");  // keeps the loads in front of the lookups below
 
-    const long long p = (long long)token + (long long)padding_offset[token];
+    const long long p = (long long)token + (long long)read_only_i32(padding_offset, (int)token);
     if (p < 0 || p >= (long long)positions) return;  // workgroup-uniform
     unsigned b, s;
     seq.divmod((unsigned)p, b, s);
@@ -415,7 +405,7 @@ __global__ __launch_bounds__(512) void qkv_rope_lean_f16(
     __shared__ float2 cs[4][16][2];
     if (rotates) {
         if (tid < 64) {
-            const float2 coef = rope_coefficients(history_length[b] + (int)s, my_divisor);
+            const float2 coef = rope_coefficients(read_only_i32(history_length, (int)b) + (int)s, my_divisor);
             const unsigned g = tid >> 3, e = tid & 7u;  // pair tid = element e of column group g
             cs[e >> 1][g][e & 1u] = make_float2(coef.x, -coef.y);  // lower half row: c x - s partner
             cs[e >> 1][g + 8][e & 1u] = coef;                      // upper half row: c x + s partner
@@ -495,8 +485,8 @@ __global__ __launch_bounds__(512) void qkv_rope_lean64_f16(
     // loads above (vector memory returns in issue order, so a vector load of the padding offset would only
     // come back behind the rows, and the first wave's evaluation with it).
     const unsigned tok_a = blockIdx.x * 2u, tok_b = tok_a + 1u;
-    const long long p_a = (long long)tok_a + (long long)padding_offset[tok_a];
-    const long long p_b = tok_b < token_num ? (long long)tok_b + (long long)padding_offset[tok_b] : -1;
+    const long long p_a = (long long)tok_a + (long long)read_only_i32(padding_offset, (int)tok_a);
+    const long long p_b = tok_b < token_num ? (long long)tok_b + (long long)read_only_i32(padding_offset, (int)tok_b) : -1;
     const bool ok_a = p_a >= 0 && p_a < (long long)positions, ok_b = p_b >= 0 && p_b < (long long)positions;
     unsigned b_a = 0, s_a = 0, b_b = 0, s_b = 0;
     if (ok_a) seq.divmod((unsigned)p_a, b_a, s_a);
@@ -510,7 +500,7 @@ __global__ __launch_bounds__(512) void qkv_rope_lean64_f16(
     if (blockIdx.y * 32u < head_num + kv_head_num) {  // workgroup-uniform: some wave here rotates
         if (tid < 64) {
             // b_a / b_b are 0 for a token without a position: both loads unconditional, so they overlap
-            const int h_a = history_length[b_a], h_b = history_length[b_b];
+            const int h_a = read_only_i32(history_length, (int)b_a), h_b = read_only_i32(history_length, (int)b_b);
             const int t_a = h_a + (int)s_a, t_b = h_b + (int)s_b;
             const float2 coef = rope_coefficients((tid & 32u) ? t_b : t_a, my_divisor);
             const unsigned d = tid & 31u, gg = d >> 3, e = d & 7u;  // pair d = element e of column group gg
@@ -600,11 +590,11 @@ __global__ __launch_bounds__(kBlock) void qkv_rope_generic(
     const int32_t* history_length, int batch, int seq_len, int head_num, int kv_head_num,
     int head_size, int half_rot, RopeDivisors tab, KvAppend<T> ap) {
     const int token = blockIdx.x;
-    const long long p = (long long)token + (long long)padding_offset[token];
+    const long long p = (long long)token + (long long)read_only_i32(padding_offset, (int)token);
     if (p < 0 || p >= (long long)batch * (long long)seq_len) return;
     const int b = (int)(p / seq_len);
     const int s = (int)(p % seq_len);
-    const int timestep = history_length[b] + s;
+    const int timestep = read_only_i32(history_length, b) + s;
     const long long cache_row = append_row(ap, history_length, b, s);
     const int half = head_size / 2;
     const int qkv_heads = head_num + 2 * kv_head_num;
