@@ -19,7 +19,7 @@
 //   out      = act x Wdown^T                                GEMM
 //   launchFusedAddBiasResidualRMSNorm(residual, out, down-bias, next layer's attn_norm)
 //
-// Every memory-bound step is one of this library's launch* entry points; the five dense GEMMs and the
+// Every memory-bound step is one of this library's launch* entry points; the four dense GEMMs and the
 // two batched attention GEMMs are hipBLASLt calls made here; the softmax between them is a plain
 // kernel of this file's own (attention is not one of the optimised kernels of this library).
 // Everything runs on the null stream, as the reference's launchers do.
