@@ -137,3 +137,21 @@ def rope_pair_radius(qkv, bias):
     half = hs // 2
     rad = np.sqrt(x[..., :half] ** 2 + x[..., half:] ** 2)
     return np.concatenate([rad, rad], axis=-1)
+
+
+def reference_mover_configurations():
+    """The inputs of the reference's own programs for the two cache movers
+    (tests/unittests/test_concat_kv.cu:16-75, test_repeat_kv.cu:15-56).  Those programs print their results
+    for inspection and state no expected values; the expectations here follow from the kernels' definitions
+    (concat_past_kv.cu:7-39, repeat_kv.cu:10-50) by hand."""
+    # append: batch 1, 2 kv heads, 16 query positions of 8 elements, cache rows of 32 positions, source = 1,
+    # 16 valid tokens behind a history of 1  =>  cache rows 1..16 of both heads become 1, nothing else changes
+    k_src = np.ones((1, 2, 16, 8), np.float32)
+    cache = np.full((1, 1, 2, 32, 8), -9.0, np.float32)
+    expect_cache = cache.copy()
+    expect_cache[0, 0, :, 1:17, :] = 1.0
+    # broadcast: 2 layers, batch 1, 2 heads = 2 kv heads, cache rows of 4 positions of 2 elements holding their own
+    # flat index, context 2, 2 key positions, layer 0  =>  head 0 reads elements 0..3, head 1 elements 8..11
+    src_cache = np.arange(2 * 1 * 2 * 4 * 2, dtype=np.float32).reshape(2, 1, 2, 4, 2)
+    expect_rep = np.array([[[[0, 1], [2, 3]], [[8, 9], [10, 11]]]], np.float32)
+    return k_src, cache, expect_cache, src_cache, expect_rep

@@ -4,7 +4,8 @@ import numpy as np
 import pytest
 import torch
 
-from helpers import assert_f16_close, assert_f32_close, padding_offsets_np, rope_pair_radius
+from helpers import (assert_f16_close, assert_f32_close, padding_offsets_np, reference_mover_configurations,
+                     rope_pair_radius)
 
 pytestmark = pytest.mark.gpu
 NP2T = {np.float16: torch.float16, np.float32: torch.float32}
@@ -206,3 +207,17 @@ def test_fallback_copy_units_through_raw_pointers(isp, shift):
     for b in range(batch):
         assert np.array_equal(got[b, :, :ctx[b]], kc_now[b, :, :ctx[b]])
         assert (got[b, :, ctx[b]:] == 7).all()
+
+
+def test_kv_cache_movers_on_the_reference_configurations(isp):
+    print("[case] kv movers on the reference programs' configurations", flush=True)
+    k_src, cache, expect_cache, src_cache, expect_rep = reference_mover_configurations()
+    d = lambda a: torch.from_numpy(a).cuda()
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device="cuda")
+    kc, vc = d(cache.copy()), d(cache.copy())
+    isp.concat_kv_cache(d(k_src), d(k_src.copy()), 0, i32([16]), i32([1]), kc, vc)
+    assert np.array_equal(kc.cpu().numpy(), expect_cache) and np.array_equal(vc.cpu().numpy(), expect_cache)
+    kd = torch.full((1, 2, 2, 2), -3.0, device="cuda")
+    vd = kd.clone()
+    isp.repeat_kv_cache(d(src_cache), d(src_cache.copy()), i32([2]), 0, kd, vd)
+    assert np.array_equal(kd.cpu().numpy(), expect_rep) and np.array_equal(vd.cpu().numpy(), expect_rep)

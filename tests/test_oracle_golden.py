@@ -141,3 +141,11 @@ def test_qkv_rope_float64_fixture(oracle, f64):
     w = f64["qkv_written"]
     assert np.all(q[~w[:, None, :].repeat(hn, 1)] == 0.0)
     assert np.all(v[~w[:, None, :].repeat(kvn, 1)] == 0.0)
+
+
+def test_reference_mover_configurations(oracle):
+    """The configurations of the reference's own programs for the KV-cache append and broadcast."""
+    from helpers import reference_mover_configurations
+    k_src, cache, expect_cache, src_cache, expect_rep = reference_mover_configurations()
+    assert np.array_equal(oracle.concat_kv(k_src, cache, 0, [16], [1]), expect_cache)
+    assert np.array_equal(oracle.repeat_kv(src_cache, 0, [2], 2, 2), expect_rep)
