@@ -482,16 +482,19 @@ def context_layer_record(torch, steps, warmup, stream):
             "note": "library kernels via the C ABI; GEMMs and attention are torch library calls"}
 
 
-def context_layer_cpp_record(torch, steps, warmup):
+def context_layer_cpp_record(torch, steps, warmup, layers=0):
     """The same layer through the C++ layer class (launch* kernels + hipBLASLt GEMMs called directly, padded
-    batched attention): runs build/bin/bench_context_layer in a child process and returns its JSON record."""
+    batched attention): runs build/bin/bench_context_layer in a child process and returns its JSON record.
+    With `layers` > 0: the whole stack of that many layers (LlamaContextDecoder, build/bin/bench_context_decoder)."""
     import subprocess
-    exe = os.path.join(ROOT, "build", "bin", "bench_context_layer")
+    name = "bench_context_decoder" if layers else "bench_context_layer"
+    exe = os.path.join(ROOT, "build", "bin", name)
     if not os.path.exists(exe):
-        return {"error": "build/bin/bench_context_layer is missing (python -m inferspore_amd.build)"}
+        return {"error": "build/bin/%s is missing (python -m inferspore_amd.build)" % name}
     lens = [str(int(v)) for v in bench_lengths(torch).tolist()]
+    counts = [str(layers), "5", "2"] if layers else [str(max(10, steps // 10)), str(max(3, warmup // 4))]
     try:
-        p = subprocess.run([exe, str(max(10, steps // 10)), str(max(3, warmup // 4)), "512"] + lens,
+        p = subprocess.run([exe] + counts + ["512"] + lens,
                            stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=300)
         lines = [l for l in p.stdout.splitlines() if l.startswith("{")]
         if p.returncode != 0 or not lines:
@@ -836,6 +839,7 @@ def main():
         layer["library_kernels_share"] = est / layer["ms_per_layer"]
         config["context_layer"] = layer
         config["context_layer_cpp"] = context_layer_cpp_record(torch, a.steps, a.warmup)
+        config["context_decoder_cpp"] = context_layer_cpp_record(torch, a.steps, a.warmup, layers=32)
         config["decode_sequence"] = decode_sequence_record(torch, stream)
     if not a.kernels_only:
         # cache-resident rates (one buffer set, no rotation): the hot-path configurations by default, every

@@ -3,9 +3,9 @@
 // reference; HIP runtime underneath.
 #include "src/weights/llama/layer_weights.h"
 
+#include <algorithm>
 #include <cmath>
 #include <cstdint>
-#include <vector>
 
 #include "src/utils/macro.h"
 
@@ -18,22 +18,29 @@ T* device_array(size_t n) {
     return p;
 }
 
-inline float to_storage(float x, float*) { return x; }
-inline half to_storage(float x, half*) { return __float2half(x); }
+__device__ inline void to_storage(float x, float* p) { *p = x; }
+__device__ inline void to_storage(float x, half* p) { *p = __float2half(x); }
 
-// value i of stream `tag`: a fixed integer hash mapped to [-scale, scale) (+ shift)
+// value i of stream `tag`: a fixed integer hash mapped to [-scale, scale) (+ shift); filled on the device
+// (a 7B-shaped layer holds 200 M weights)
 template <typename T>
-void fill(T* dst, size_t n, uint32_t tag, float scale, float shift) {
-    std::vector<T> h(n);
-    for (size_t i = 0; i < n; i++) {
+__global__ void fill_kernel(T* dst, size_t n, uint32_t tag, float scale, float shift) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
         uint32_t x = (uint32_t)i * 2654435761u + tag * 40503u + 12345u;
         x ^= x >> 15;
         x *= 2246822519u;
         x ^= x >> 13;
         const float u = (float)(x >> 8) * (1.0f / 16777216.0f) - 0.5f;  // [-0.5, 0.5)
-        h[i] = to_storage(shift + 2.0f * scale * u, static_cast<T*>(nullptr));
+        to_storage(shift + 2.0f * scale * u, dst + i);
     }
-    CHECK(hipMemcpy(dst, h.data(), n * sizeof(T), hipMemcpyHostToDevice));
+}
+
+template <typename T>
+void fill(T* dst, size_t n, uint32_t tag, float scale, float shift) {
+    if (n == 0) return;
+    const unsigned blocks = (unsigned)std::min<size_t>((n + 255) / 256, 65536);
+    hipLaunchKernelGGL(fill_kernel<T>, dim3(blocks), dim3(256), 0, nullptr, dst, n, tag, scale, shift);
+    CHECK(hipGetLastError());
 }
 
 }  // namespace
@@ -92,6 +99,7 @@ void LlamaLayerWeight<T>::loadWeights() {
         fill(self_attn_weight.qkv.bias, (size_t)qkv_out, 7, 0.02f, 0.0f);
         fill(self_attn_weight.output.bias, (size_t)hidden_units, 8, 0.02f, 0.0f);
     }
+    CHECK(hipDeviceSynchronize());
 }
 
 template class LlamaLayerWeight<float>;

@@ -6,11 +6,13 @@
 //
 //   test_context_layer <f32|f16> <directory> [head_num kv_head_num head_size inter_size]
 #include <cstdio>
+#include <memory>
 #include <numeric>
 #include <string>
 
 #include "src/kernels/cal_paddingoffset.h"
 #include "src/kernels/rmsnorm.h"
+#include "src/layers/decoder/context_decoder.h"
 #include "src/layers/decoder/context_decoder_layer.h"
 #include "src/memory/allocator/hip_allocator.h"
 #include "test_util.h"
@@ -165,6 +167,111 @@ static int run(const std::string& dir, int head_num, int kv_heads, int head_size
     double err_k = 0;
     for (size_t i = 0; i < ka.size(); i++) err_k = std::max(err_k, std::fabs((double)Host<T>::from(ka[i]) - Host<T>::from(kb[i])));
     EXPECT(err_k <= tol * 8.0, "two turns: cached keys differ by %g", err_k);
+
+    // ---- case 3: the decoder stack equals its layers called one by one
+    {
+        const int stack_layers = 3;
+        std::vector<std::unique_ptr<LlamaLayerWeight<T>>> owned;
+        std::vector<LlamaLayerWeight<T>*> ws;
+        for (int l = 0; l < stack_layers; l++) {
+            owned.emplace_back(new LlamaLayerWeight<T>(head_num, kv_heads, head_size, inter, getWeightType<T>(), l == 1));
+            owned.back()->loadWeights();
+            // distinct norms per layer, so that a layer picking the wrong "next" norm shows
+            auto g1 = randn<T>(hidden, 0.25f, gen, 1.0f), g2 = randn<T>(hidden, 0.25f, gen, 1.0f);
+            CHECK(hipMemcpy(owned.back()->attn_norm_weight.gamma, g1.data(), hidden * sizeof(S), hipMemcpyHostToDevice));
+            CHECK(hipMemcpy(owned.back()->ffn_norm_weight.gamma, g2.data(), hidden * sizeof(S), hipMemcpyHostToDevice));
+            ws.push_back(owned.back().get());
+        }
+        const std::vector<int> l3 = {7, 16, 3}, h3 = {0, 0, 0};
+        Batch<T> b3(l3, h3, max_q);
+        auto emb = randn<T>((size_t)b3.tokens * hidden, 1.0f, gen);
+        const size_t n = emb.size(), cache3 = (size_t)stack_layers * b3.batch * kv_heads * max_seq * head_size;
+        // by hand
+        T* r = (T*)to_device(emb);
+        T* nrm = (T*)to_device(std::vector<S>(n));
+        T* o = (T*)to_device(std::vector<S>(n));
+        T* kc1 = (T*)to_device(std::vector<S>(cache3));
+        T* vc1 = (T*)to_device(std::vector<S>(cache3));
+        {
+            const DataType dt = getTensorType<T>();
+            CHECK(hipMemcpy(nrm, r, n * sizeof(T), hipMemcpyDeviceToDevice));
+            TensorWrapper<T> first(Device::GPU, dt, {b3.tokens, hidden}, nrm);
+            launchRMSNorm(&first, ws[0]->attn_norm_weight, 1e-5f);
+            T *from = nrm, *to = o;
+            for (int l = 0; l < stack_layers; l++) {
+                TensorWrapper<T> in(Device::GPU, dt, {b3.tokens, hidden}, from), res(Device::GPU, dt, {b3.tokens, hidden}, r);
+                TensorWrapper<T> out_t(Device::GPU, dt, {b3.tokens, hidden}, to);
+                TensorWrapper<int> po(Device::GPU, getTensorType<int>(), {b3.batch, b3.max_q}, b3.padding_offset);
+                TensorWrapper<int> hl(Device::GPU, getTensorType<int>(), {b3.batch}, b3.hist);
+                TensorWrapper<int> il(Device::GPU, getTensorType<int>(), {b3.batch}, b3.lens);
+                TensorWrapper<int> cl(Device::GPU, getTensorType<int>(), {b3.batch}, b3.ctx);
+                int lv = l;
+                TensorWrapper<int> lid(Device::CPU, getTensorType<int>(), {1}, &lv);
+                TensorWrapper<T> kc(Device::GPU, dt, {stack_layers, b3.batch, kv_heads, max_seq, head_size}, kc1);
+                TensorWrapper<T> vc(Device::GPU, dt, {stack_layers, b3.batch, kv_heads, max_seq, head_size}, vc1);
+                TensorMap li{{"decoder_input", &in}, {"decoder_residual", &res}, {"padding_offset", &po}, {"history_length", &hl},
+                             {"input_length", &il}, {"context_length", &cl}, {"layer_id", &lid}};
+                TensorMap lo{{"decoder_output", &out_t}, {"all_k_cache", &kc}, {"all_v_cache", &vc}};
+                LLaMAAttentionDynParams dyn;
+                dyn.batch_size = b3.batch, dyn.num_tokens = b3.tokens, dyn.max_q_len = b3.max_q, dyn.max_k_len = b3.max_k;
+                dyn.num_layers = stack_layers;
+                layer.forward(li, *ws[l], l + 1 < stack_layers ? ws[l + 1]->attn_norm_weight : next, lo, dyn);
+                std::swap(from, to);
+            }
+            CHECK(hipDeviceSynchronize());
+            if (from != o) CHECK(hipMemcpy(o, from, n * sizeof(T), hipMemcpyDeviceToDevice));
+        }
+        // through the stack
+        T* e2 = (T*)to_device(emb);
+        T* o2 = (T*)to_device(std::vector<S>(n));
+        T* kc2 = (T*)to_device(std::vector<S>(cache3));
+        T* vc2 = (T*)to_device(std::vector<S>(cache3));
+        {
+            const DataType dt = getTensorType<T>();
+            LlamaContextDecoder<T> decoder(head_num, kv_heads, head_size, inter, stack_layers, params, 1e-5f, &allocator);
+            TensorWrapper<T> in(Device::GPU, dt, {b3.tokens, hidden}, e2), out_t(Device::GPU, dt, {b3.tokens, hidden}, o2);
+            TensorWrapper<int> hl(Device::GPU, getTensorType<int>(), {b3.batch}, b3.hist);
+            TensorWrapper<int> il(Device::GPU, getTensorType<int>(), {b3.batch}, b3.lens);
+            TensorWrapper<int> cl(Device::GPU, getTensorType<int>(), {b3.batch}, b3.ctx);
+            TensorWrapper<T> kc(Device::GPU, dt, {stack_layers, b3.batch, kv_heads, max_seq, head_size}, kc2);
+            TensorWrapper<T> vc(Device::GPU, dt, {stack_layers, b3.batch, kv_heads, max_seq, head_size}, vc2);
+            TensorMap di{{"decoder_input", &in}, {"history_length", &hl}, {"input_length", &il}, {"context_length", &cl}};
+            TensorMap dout{{"decoder_output", &out_t}, {"all_k_cache", &kc}, {"all_v_cache", &vc}};
+            LLaMAAttentionDynParams dyn;
+            dyn.batch_size = b3.batch, dyn.num_tokens = b3.tokens, dyn.max_q_len = b3.max_q, dyn.max_k_len = b3.max_k;
+            dyn.num_layers = stack_layers;
+            decoder.forward(di, ws, next, dout, dyn);
+            CHECK(hipDeviceSynchronize());
+            auto kept = to_host((S*)e2, n);
+            EXPECT(std::memcmp(kept.data(), emb.data(), n * sizeof(S)) == 0, "the stack must leave decoder_input unchanged");
+            std::vector<LlamaLayerWeight<T>*> too_few(ws.begin(), ws.begin() + 2);
+            EXPECT(throws([&] { decoder.forward(di, too_few, next, dout, dyn); }), "a missing layer's weights must throw");
+        }
+        // the two engines choose their GEMM algorithms by measurement, each for itself, so the comparison allows
+        // for a different summation order inside the GEMMs
+        auto a = to_host((S*)o, n), b = to_host((S*)o2, n);
+        auto worst = [](const std::vector<S>& u, const std::vector<S>& w, double& scale) {
+            double err = 0;
+            scale = 0;
+            for (size_t i = 0; i < u.size(); i++) {
+                scale = std::max(scale, std::fabs((double)Host<T>::from(u[i])));
+                err = std::max(err, std::fabs((double)Host<T>::from(u[i]) - Host<T>::from(w[i])));
+            }
+            return err;
+        };
+        double sc = 0;
+        const double tol3 = std::is_same<T, float>::value ? 3e-4 : 3e-2;
+        const double eo = worst(a, b, sc);
+        EXPECT(eo <= tol3 * sc, "decoder stack: output differs from the layers called by hand by %g (scale %g)", eo, sc);
+        auto ka3 = to_host((S*)kc1, cache3), kb3 = to_host((S*)kc2, cache3), va3 = to_host((S*)vc1, cache3), vb3 = to_host((S*)vc2, cache3);
+        const double ek = worst(ka3, kb3, sc);
+        EXPECT(ek <= tol3 * sc, "decoder stack: cached keys differ by %g (scale %g)", ek, sc);
+        const double ev = worst(va3, vb3, sc);
+        EXPECT(ev <= tol3 * sc, "decoder stack: cached values differ by %g (scale %g)", ev, sc);
+        double peak = 0;
+        for (size_t i = 0; i < n; i++) peak = std::max(peak, std::fabs((double)Host<T>::from(b[i])));
+        EXPECT(peak > 0.1 && peak < 100.0, "decoder stack: implausible output scale %g", peak);
+    }
 
     // ---- the layer rejects tensors that do not fit
     {
