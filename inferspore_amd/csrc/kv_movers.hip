@@ -46,14 +46,15 @@ static SegSplit make_split(unsigned seg_vec) {
 
 // dst[token, h, :] = src[b, h, s, :],  token + padding_offset[token] = b * seq_len + s.
 // grid = tokens * chunks, a chunk being 256 vectors of the token's heads*seg_vec vectors
-__global__ __launch_bounds__(kBlock) void transpose_remove_padding_vec(
+template <int BLOCK>
+__global__ __launch_bounds__(BLOCK) void transpose_remove_padding_vec(
     const char* __restrict__ src, const int32_t* __restrict__ padding_offset, char* __restrict__ dst,
     unsigned positions, int head_num, FastDiv seq, SegSplit sp, FastDiv chunks) {
     const unsigned seg_vec = sp.seg_vec;
     const unsigned seq_len = seq.d;
     unsigned token, chunk;
     chunks.divmod(blockIdx.x, token, chunk);
-    const unsigned vi = chunk * kBlock + threadIdx.x;  // vector index inside the token's row
+    const unsigned vi = chunk * BLOCK + threadIdx.x;  // vector index inside the token's row
     const unsigned row_vec = (unsigned)head_num * seg_vec;
     if (vi >= row_vec) return;
     const long long p = (long long)token + (long long)read_only_i32(padding_offset, (int)token);
@@ -202,16 +203,26 @@ static int transpose_remove_padding(const void* src, const int32_t* padding_offs
     ISP_REQUIRE_PTR(padding_offset);
     ISP_REQUIRE_PTR(dst);
     const size_t seg = (size_t)head_size * elem;
-    const size_t chunks = ((size_t)head_num * (seg / 16) + kBlock - 1) / kBlock;
+    const size_t row_vec = (size_t)head_num * (seg / 16);
+    // one 512-thread workgroup per token when a token's row is exactly that (32 heads of 256 bytes): 9.54
+    // against 9.79 us; with two such workgroups per token (64 heads) 256 threads stay 0.7 % ahead.  The knob
+    // of the cache movers overrides.
+    const int knob = tuning(ISP_TUNE_MOVER_BLOCK_THREADS);
+    const int blk = (knob == 256 || knob == 512) ? knob : (row_vec == 512 ? 512 : 256);
+    const size_t chunks = (row_vec + blk - 1) / blk;
     // the vector kernel keeps padded positions in 32 bits and divides with a multiply-high
     if (seg % 16 == 0 && aligned16(src) && aligned16(dst) && chunks * (size_t)token_num <= 0x7fffffffull &&
         (unsigned long long)batch * (unsigned long long)seq_len <= 0x7fffffffull) {
         const unsigned seg_vec = (unsigned)(seg / 16);
         dim3 grid((unsigned)(chunks * (size_t)token_num));
-        hipLaunchKernelGGL(transpose_remove_padding_vec, grid, dim3(kBlock), 0, s,
-                           static_cast<const char*>(src), padding_offset, static_cast<char*>(dst),
-                           (unsigned)batch * (unsigned)seq_len, head_num, make_fastdiv((unsigned)seq_len),
-                           make_split(seg_vec), make_fastdiv((unsigned)chunks));
+#define ISP_LAUNCH_TRANSPOSE(B)                                                                     \
+    hipLaunchKernelGGL(transpose_remove_padding_vec<B>, grid, dim3(B), 0, s,                         \
+                       static_cast<const char*>(src), padding_offset, static_cast<char*>(dst),       \
+                       (unsigned)batch * (unsigned)seq_len, head_num, make_fastdiv((unsigned)seq_len), \
+                       make_split(seg_vec), make_fastdiv((unsigned)chunks))
+        if (blk == 512) ISP_LAUNCH_TRANSPOSE(512);
+        else ISP_LAUNCH_TRANSPOSE(256);
+#undef ISP_LAUNCH_TRANSPOSE
     } else {
         const dim3 grid((unsigned)token_num), block(kBlock);
 #define ISP_LAUNCH_UNITS(U)                                                                        \

@@ -213,6 +213,32 @@ def test_kv_movers_every_workgroup_size(isp):
         assert all(np.array_equal(a, b) for a, b in zip(got, base))
 
 
+def test_transpose_out_every_workgroup_size(isp):
+    """32 heads of 256 bytes take one 512-thread workgroup per token by default, everything else 256-thread
+    ones; both sizes must move the same bytes for either shape."""
+    from inferspore_amd import capi
+    for heads in (32, 40):
+        batch, seq, hs = 3, 10, 128
+        lens = np.array([10, 3, 7], np.int32)
+        tokens = int(lens.sum())
+        g = torch.Generator(device="cuda").manual_seed(heads)
+        src = torch.randn((batch, heads, seq, hs), device="cuda", generator=g).half()
+        po = torch.zeros((batch, seq), dtype=torch.int32, device="cuda")
+        po.view(-1)[:tokens] = torch.from_numpy(np.repeat(np.cumsum(seq - lens) - (seq - lens), lens).astype(np.int32)).cuda()
+
+        def run():
+            out = torch.full((tokens, heads, hs), -4.0, dtype=torch.float16, device="cuda")
+            isp.transpose_out_remove_padding(src, po, out)
+            return out.cpu().numpy()
+
+        base = run()
+        expect = np.concatenate([src[b, :, :n].permute(1, 0, 2).cpu().numpy() for b, n in enumerate(lens)])
+        assert np.array_equal(base, expect)
+        for block in (256, 512):
+            say("transpose-out, %d heads, %d-thread workgroups" % (heads, block))
+            assert np.array_equal(with_knobs({capi.TUNE_MOVER_BLOCK_THREADS: block}, run), base)
+
+
 def test_kv_movers_more_rows_than_a_grid_dimension_holds(isp):
     """A decode step of a large batch has more (sequence, head) rows than the 65535 a grid's second
     dimension can count; the movers index their workgroups linearly, so it must simply work."""
