@@ -563,6 +563,19 @@ def decode_sequence_record(torch, stream):
             out[tag + "eager_us_per_step"] = eager_us
             out[tag + "graph_replay_us_per_step"] = timed(graph.replay, 200)
             out[tag + "kernels_per_step"] = n_kernels
+    # the fused step from a C++ caller (no ctypes call per launch)
+    import subprocess
+    exe = os.path.join(ROOT, "build", "bin", "bench_decode_sequence")
+    if os.path.exists(exe):
+        try:
+            p = subprocess.run([exe, "500"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=120)
+            lines = [l for l in p.stdout.splitlines() if l.startswith("{")]
+            if p.returncode == 0 and lines:
+                out.update(json.loads(lines[-1]))
+            else:
+                out["cpp_error"] = p.stdout[-300:]
+        except (OSError, subprocess.SubprocessError, ValueError) as e:
+            out["cpp_error"] = str(e)
     return out
 
 
