@@ -42,6 +42,17 @@
 
 namespace isp_layers {
 class GemmEngine;  // hipBLASLt handle, workspace and per-shape algorithm cache
+
+// The layer's attention softmax, in place on scores [batch, head_num, max_q_len, max_k_len] (device memory,
+// null stream): row (b, h, q) becomes softmax(scale * scores) over the keys that query q may see -- key
+// positions <= history_length[b] + q and < context_length[b] -- and exactly zero elsewhere; rows of padded
+// queries (q >= input_length[b]) become zero.  The mask is computed from the three [batch] length arrays
+// instead of being read from a [batch, q, k] tensor (src/kernels/build_casual_mask.cu:5-42,
+// attn_softmax_kernel.cu:50-125).  Instantiated for float and half.
+template <typename T>
+void launch_masked_scaled_softmax(T* scores, const int* history_length, const int* input_length,
+                                  const int* context_length, int batch, int head_num, int max_q_len,
+                                  int max_k_len, float scale);
 }
 
 template <typename T>

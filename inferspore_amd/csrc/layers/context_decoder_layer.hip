@@ -238,61 +238,102 @@ __global__ __launch_bounds__(256) void masked_scaled_softmax(T* scores, const in
     }
 }
 
+// Lane exchange inside the VALU (no LDS traffic); `ctrl` is the DPP control word.
+template <int ctrl>
+__device__ __forceinline__ float lane_swap(float x) {
+    return __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(x), ctrl, 0xf, 0xf, true));
+}
+__device__ __forceinline__ float read_lane(float x, int lane) {
+    return __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(x), lane));
+}
+// Maximum / sum over the 64 lanes, the result in every lane: quad swaps and the two row mirrors fold each
+// row of 16 lanes, the four row results are combined as scalars.
+__device__ __forceinline__ float wave_max(float x) {
+    x = fmaxf(x, lane_swap<0xB1>(x));
+    x = fmaxf(x, lane_swap<0x4E>(x));
+    x = fmaxf(x, lane_swap<0x141>(x));
+    x = fmaxf(x, lane_swap<0x140>(x));
+    return fmaxf(fmaxf(read_lane(x, 0), read_lane(x, 16)), fmaxf(read_lane(x, 32), read_lane(x, 48)));
+}
+__device__ __forceinline__ float wave_total(float x) {
+    x += lane_swap<0xB1>(x);
+    x += lane_swap<0x4E>(x);
+    x += lane_swap<0x141>(x);
+    x += lane_swap<0x140>(x);
+    return (read_lane(x, 0) + read_lane(x, 16)) + (read_lane(x, 32) + read_lane(x, 48));
+}
+__device__ __forceinline__ int uniform_i32(const int* p, int i) {
+    // the lengths never change while a kernel runs: read them through the scalar cache
+    typedef const int __attribute__((address_space(4)))* constant_ints;
+    return reinterpret_cast<constant_ints>((unsigned long long)p)[i];
+}
+
 // The same, one wavefront per row with the row in registers: NVW 16-byte vectors per lane cover rows of
 // up to 64 * NVW vectors (512 * NVW fp16 keys), every element is read once and written once, vectors that
 // lie wholly behind the visible keys are not read at all, and rows of padded queries are only zeroed.
-// exp through the hardware exponential (relative error about 2^-22, far inside what the attention
-// output is compared at).  Used when max_k_len is a whole number of vectors and fits; else the kernel above.
+// The kernel is bound as much by its instruction count as by memory (a 1 KiB row per wavefront), so the
+// grid's three dimensions name (query / 4, head, batch) and no index is divided, the reductions stay in
+// the VALU, the scale is folded into the exponent -- p = 2^(x * c - max(x) * c) with c = scale * log2(e),
+// the maximum taken over the raw scores since scale > 0 -- and masked keys are set to -inf once, which the
+// hardware exponential turns into exactly 0.  That exponential has a relative error of about 2^-22, far
+// inside what the attention output is compared at.  Used when max_k_len is a whole number of vectors and
+// fits; else the kernel above.
 template <typename T, int NVW>
 __global__ __launch_bounds__(256) void masked_scaled_softmax_rows(T* scores, const int* history_length,
                                                                   const int* input_length,
-                                                                  const int* context_length, int head_num,
-                                                                  int max_q_len, int max_k_len, float scale,
-                                                                  long long rows) {
+                                                                  const int* context_length, int max_q_len,
+                                                                  int max_k_len, float scale_log2e) {
     constexpr int VEC = 16 / (int)sizeof(T);
     union Vec16 {
         uint4 raw;
         T e[VEC];
     };
     const int lane = threadIdx.x % 64;
-    const long long row_id = (long long)blockIdx.x * 4 + threadIdx.x / 64;
-    if (row_id >= rows) return;  // wave-uniform
-    const int q = (int)(row_id % max_q_len);
-    const int b = (int)(row_id / max_q_len / head_num);
+    const int q = __builtin_amdgcn_readfirstlane((int)(blockIdx.x * 4 + threadIdx.x / 64));
+    if (q >= max_q_len) return;  // wave-uniform
+    const int b = blockIdx.z;
     int visible = 0;
-    if (q < input_length[b]) {
-        visible = history_length[b] + q + 1;
-        if (visible > context_length[b]) visible = context_length[b];
-        if (visible > max_k_len) visible = max_k_len;
+    if (q < uniform_i32(input_length, b)) {
+        visible = min(min(uniform_i32(history_length, b) + q + 1, uniform_i32(context_length, b)), max_k_len);
     }
-    T* row = scores + (size_t)row_id * (size_t)max_k_len;
+    T* row = scores + (((size_t)b * gridDim.y + blockIdx.y) * (size_t)max_q_len + (size_t)q) * (size_t)max_k_len;
     const int nvec = max_k_len / VEC;
+    if (visible <= 0) {  // wave-uniform: a padded query
+#pragma unroll
+        for (int j = 0; j < NVW; j++) {
+            const int vi = lane + 64 * j;
+            if (vi < nvec) *reinterpret_cast<uint4*>(row + vi * VEC) = make_uint4(0u, 0u, 0u, 0u);
+        }
+        return;
+    }
     float x[NVW][VEC];
     float m = -INFINITY;
 #pragma unroll
     for (int j = 0; j < NVW; j++) {
-        const int vi = lane + 64 * j, k0 = vi * VEC;
+        const int k0 = (lane + 64 * j) * VEC;
+        const int left = visible - k0;  // keys of this vector that are visible, if positive (visible <= max_k_len)
         Vec16 v;
-        const bool have = vi < nvec && k0 < visible;
-        if (have) v.raw = *reinterpret_cast<const uint4*>(row + k0);
+        v.raw = make_uint4(0u, 0u, 0u, 0u);
+        if (left > 0) v.raw = *reinterpret_cast<const uint4*>(row + k0);
 #pragma unroll
         for (int e = 0; e < VEC; e++) {
-            x[j][e] = (have && k0 + e < visible) ? scale * to_float(v.e[e]) : -INFINITY;
+            x[j][e] = e < left ? to_float(v.e[e]) : -INFINITY;
             m = fmaxf(m, x[j][e]);
         }
     }
-    for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off, 64));
+    m = wave_max(m);
+    const float mc = m * scale_log2e;
     float sum = 0.0f;
 #pragma unroll
     for (int j = 0; j < NVW; j++) {
 #pragma unroll
         for (int e = 0; e < VEC; e++) {
-            x[j][e] = x[j][e] == -INFINITY ? 0.0f : __expf(x[j][e] - m);
+            x[j][e] = __builtin_amdgcn_exp2f(fmaf(x[j][e], scale_log2e, -mc));
             sum += x[j][e];
         }
     }
-    for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
-    const float inv = visible > 0 ? 1.0f / sum : 0.0f;
+    sum = wave_total(sum);
+    const float inv = 1.0f / sum;  // at least 2^0 went into the sum
 #pragma unroll
     for (int j = 0; j < NVW; j++) {
         const int vi = lane + 64 * j;
@@ -310,15 +351,17 @@ void launch_masked_scaled_softmax(T* scores, const int* history_length, const in
                                   const int* context_length, int batch, int head_num, int max_q_len,
                                   int max_k_len, float scale) {
     constexpr int VEC = 16 / (int)sizeof(T);
-    const long long rows = (long long)batch * head_num * max_q_len;
     const int nvec = max_k_len / VEC;
+    LLM_CHECK_WITH_INFO(batch > 0 && head_num > 0 && max_q_len > 0 && max_k_len > 0 && batch <= 65535 && head_num <= 65535,
+                        "attention scores of an extent no grid holds");
     const bool rows_ok = max_k_len % VEC == 0 && nvec <= 64 * 4 && (reinterpret_cast<uintptr_t>(scores) & 15u) == 0 &&
-                         (rows + 3) / 4 <= 0x7fffffffLL;
+                         scale > 0.0f;
     if (rows_ok) {
-        const dim3 grid((unsigned)((rows + 3) / 4)), block(256);
+        const dim3 grid((unsigned)((max_q_len + 3) / 4), (unsigned)head_num, (unsigned)batch), block(256);
+        const float scale_log2e = scale * 1.4426950408889634f;
 #define ISP_SOFTMAX_ROWS(N)                                                                              \
     hipLaunchKernelGGL((masked_scaled_softmax_rows<T, N>), grid, block, 0, nullptr, scores, history_length, \
-                       input_length, context_length, head_num, max_q_len, max_k_len, scale, rows)
+                       input_length, context_length, max_q_len, max_k_len, scale_log2e)
         if (nvec <= 64) ISP_SOFTMAX_ROWS(1);
         else if (nvec <= 128) ISP_SOFTMAX_ROWS(2);
         else ISP_SOFTMAX_ROWS(4);
@@ -330,6 +373,9 @@ void launch_masked_scaled_softmax(T* scores, const int* history_length, const in
     }
     CHECK(hipGetLastError());
 }
+
+template void launch_masked_scaled_softmax<float>(float*, const int*, const int*, const int*, int, int, int, int, float);
+template void launch_masked_scaled_softmax<half>(half*, const int*, const int*, const int*, int, int, int, int, float);
 
 }  // namespace isp_layers
 

@@ -273,6 +273,71 @@ static int run(const std::string& dir, int head_num, int kv_heads, int head_size
         EXPECT(peak > 0.1 && peak < 100.0, "decoder stack: implausible output scale %g", peak);
     }
 
+    // ---- case 4: the attention softmax by itself against float64, at every row width its kernels split on
+    {
+        struct Shape {
+            int batch, heads, max_q, max_k;
+        };
+        // 16: a few vectors; 100: a whole number of fp32 vectors but not of fp16 ones (the workgroup-per-row kernel);
+        // 512 / 1024 / 2048: one, two and four vectors per lane; 1032 and 2056: the last lanes idle; 5 and 7 queries:
+        // a last workgroup with idle wavefronts
+        const Shape shapes[] = {{3, 2, 5, 16}, {2, 3, 7, 100}, {2, 2, 16, 512}, {2, 1, 9, 1024}, {2, 1, 6, 1032},
+                                {1, 2, 5, 2048}, {1, 1, 4, 2056}, {1, 1, 3, 4096}};
+        for (const Shape& sh : shapes) {
+            std::vector<int> hl(sh.batch), il(sh.batch), cl(sh.batch);
+            for (int b = 0; b < sh.batch; b++) {
+                il[b] = b == 0 ? sh.max_q : 1 + (int)(gen() % (unsigned)sh.max_q);              // a ragged batch
+                hl[b] = b == 0 ? 0 : (int)(gen() % (unsigned)std::max(1, sh.max_k - il[b]));   // some with history
+                cl[b] = b == 1 ? std::max(1, hl[b] + il[b] - 1) : hl[b] + il[b];                // one context cut short
+                cl[b] = std::min(cl[b], sh.max_k);
+            }
+            const size_t n = (size_t)sh.batch * sh.heads * sh.max_q * sh.max_k;
+            auto in = randn<T>(n, 8.0f, gen);   // scaled by 1/sqrt(128): exponents spread over +-3
+            T* d = (T*)to_device(in);
+            int* d_hl = (int*)to_device(hl);
+            int* d_il = (int*)to_device(il);
+            int* d_cl = (int*)to_device(cl);
+            const float scale = 0.08838834764831845f;
+            isp_layers::launch_masked_scaled_softmax(d, d_hl, d_il, d_cl, sh.batch, sh.heads, sh.max_q, sh.max_k, scale);
+            CHECK(hipDeviceSynchronize());
+            auto out = to_host((S*)d, n);
+            double worst = 0, worst_sum = 0;
+            long long leaked = 0;
+            for (int b = 0; b < sh.batch; b++)
+                for (int h = 0; h < sh.heads; h++)
+                    for (int q = 0; q < sh.max_q; q++) {
+                        const size_t base = (((size_t)b * sh.heads + h) * sh.max_q + q) * sh.max_k;
+                        int visible = 0;
+                        if (q < il[b]) visible = std::min(std::min(hl[b] + q + 1, cl[b]), sh.max_k);
+                        double m = -1e300, sum = 0, got_sum = 0;
+                        for (int k = 0; k < visible; k++) m = std::max(m, (double)scale * Host<T>::from(in[base + k]));
+                        for (int k = 0; k < visible; k++) sum += std::exp((double)scale * Host<T>::from(in[base + k]) - m);
+                        for (int k = 0; k < sh.max_k; k++) {
+                            const double got = Host<T>::from(out[base + k]);
+                            if (k >= visible) {
+                                leaked += got != 0.0;
+                                continue;
+                            }
+                            const double want = std::exp((double)scale * Host<T>::from(in[base + k]) - m) / sum;
+                            worst = std::max(worst, std::fabs(got - want) / (std::is_same<T, float>::value ? want : std::max(want, 1.0 / 1024)));
+                            got_sum += got;
+                        }
+                        if (visible > 0) worst_sum = std::max(worst_sum, std::fabs(got_sum - 1.0));
+                    }
+            // fp32: the hardware exponential's 2^-22 and the rounding of the scaled difference; fp16: one rounding of the result
+            const double tol = std::is_same<T, float>::value ? 4e-6 : 6e-4;
+            EXPECT(leaked == 0, "softmax %dx%dx%dx%d: %lld masked probabilities are not exactly zero", sh.batch, sh.heads,
+                   sh.max_q, sh.max_k, leaked);
+            EXPECT(worst <= tol, "softmax %dx%dx%dx%d: relative error %g", sh.batch, sh.heads, sh.max_q, sh.max_k, worst);
+            EXPECT(worst_sum <= (std::is_same<T, float>::value ? 1e-5 : 4e-3), "softmax %dx%dx%dx%d: a row sums to 1 %+g",
+                   sh.batch, sh.heads, sh.max_q, sh.max_k, worst_sum);
+            CHECK(hipFree(d));
+            CHECK(hipFree(d_hl));
+            CHECK(hipFree(d_il));
+            CHECK(hipFree(d_cl));
+        }
+    }
+
     // ---- the layer rejects tensors that do not fit
     {
         Batch<T> b2(lens, hist, max_q);
