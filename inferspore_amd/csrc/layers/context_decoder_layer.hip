@@ -13,6 +13,7 @@
 #include <map>
 #include <string>
 #include <tuple>
+#include <utility>
 #include <vector>
 #include <algorithm>
 
@@ -111,9 +112,9 @@ private:
                                                        sizeof(offset)));
     }
 
-    // Milliseconds per product with `algo` (two untimed runs, then the mean of five); negative if it fails.
+    // Milliseconds per product with `algo` (two untimed runs, then the mean of `runs`); negative if it fails.
     float time_algo(const Plan& p, const hipblasLtMatmulAlgo_t& algo, const void* a, const void* w, void* c,
-                    float alpha) {
+                    float alpha, int runs = 5) {
         const float beta = 0.0f;
         hipEvent_t e0, e1;
         if (hipEventCreate(&e0) != hipSuccess) return -1.0f;
@@ -123,14 +124,14 @@ private:
         }
         float ms = -1.0f;
         bool ok = true;
-        for (int i = 0; i < 7 && ok; i++) {
+        for (int i = 0; i < 2 + runs && ok; i++) {
             if (i == 2) ok = hipEventRecord(e0, nullptr) == hipSuccess;
             ok = ok && hipblasLtMatmul(handle_, p.desc, &alpha, w, p.w, a, p.a, &beta, c, p.c, c, p.c, &algo,
                                        workspace_, kWorkspaceBytes, nullptr) == HIPBLAS_STATUS_SUCCESS;
         }
         if (ok && hipEventRecord(e1, nullptr) == hipSuccess && hipEventSynchronize(e1) == hipSuccess &&
             hipEventElapsedTime(&ms, e0, e1) == hipSuccess)
-            ms /= 5.0f;
+            ms /= (float)runs;
         else
             ms = -1.0f;
         (void)hipGetLastError();
@@ -165,12 +166,20 @@ private:
         int best = 0;
         float best_ms = -1.0f;
         if (autotune_ && count > 1) {
+            // a first pass over every proposal, then the four fastest again over more runs: differences of a
+            // per cent or two between the leaders are inside the noise of five runs
+            std::vector<std::pair<float, int>> timed;
             for (int i = 0; i < count; i++) {
                 if (found[i].workspaceSize > kWorkspaceBytes) continue;
                 const float ms = time_algo(p, found[i].algo, a, w, c, alpha);
+                if (ms >= 0.0f) timed.emplace_back(ms, i);
+            }
+            std::sort(timed.begin(), timed.end());
+            for (size_t j = 0; j < timed.size() && j < 4; j++) {
+                const float ms = timed.size() > 1 ? time_algo(p, found[timed[j].second].algo, a, w, c, alpha, 20) : timed[j].first;
                 if (ms >= 0.0f && (best_ms < 0.0f || ms < best_ms)) {
                     best_ms = ms;
-                    best = i;
+                    best = timed[j].second;
                 }
             }
         }
