@@ -105,3 +105,4 @@ def test_layers_library_exports_the_layer_classes():
         assert "LlamaContextDecoderLayer<%s>::forward(" % t in syms
         assert "LlamaContextDecoderLayer<%s>::allocForForward(" % t in syms
         assert "LlamaLayerWeight<%s>::loadWeights()" % t in syms
+        assert "isp_layers::launch_masked_scaled_softmax<%s>(" % t in syms
