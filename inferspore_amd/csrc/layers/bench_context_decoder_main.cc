@@ -84,7 +84,7 @@ int main(int argc, char** argv) {
                     "\"max_q_len\": %d, \"ms_per_forward\": %.4f, \"ms_per_layer\": %.4f, \"prefill_tokens_per_s\": %.1f, "
                     "\"iterations\": %d, "
                     "\"note\": \"C++ LlamaContextDecoder: padding offsets + first RMSNorm + the layer stack (launch* kernels, "
-                    "hipBLASLt GEMMs, padded batched attention); embedding and LM head excluded\"}\n",
+                    "hipBLASLt GEMMs, attention fused on the matrix cores unless ISP_LAYERS_ATTENTION=padded); embedding and LM head excluded\"}\n",
                     layers, tokens, batch, max_q, ms, ms / layers, tokens / (ms * 1e-3), iterations);
     } catch (const std::exception& e) {
         std::printf("exception: %s\n", e.what());

@@ -4,6 +4,7 @@
 // null stream around all iterations.  Used by bench.py for its `context_layer_cpp` record.
 #include <cstdio>
 #include <cstdlib>
+#include <cstring>
 #include <numeric>
 #include <vector>
 
@@ -17,6 +18,11 @@ static V* upload(const std::vector<V>& h) {
     CHECK(hipMalloc((void**)&d, h.size() * sizeof(V) + 16));
     CHECK(hipMemcpy(d, h.data(), h.size() * sizeof(V), hipMemcpyHostToDevice));
     return d;
+}
+
+static const char* attention_kind() {
+    const char* a = std::getenv("ISP_LAYERS_ATTENTION");
+    return a != nullptr && std::strcmp(a, "padded") == 0 ? "padded" : "fused";
 }
 
 int main(int argc, char** argv) {
@@ -87,8 +93,9 @@ int main(int argc, char** argv) {
         std::printf("{\"workload\": \"llama2_7b_context_decoder_layer_f16_cpp\", \"valid_tokens\": %d, \"batch\": %d, "
                     "\"max_q_len\": %d, \"ms_per_layer\": %.6f, \"tokens_per_s_per_layer\": %.1f, \"iterations\": %d, "
                     "\"activation_buffer_bytes\": %zu, "
-                    "\"note\": \"C++ LlamaContextDecoderLayer: launch* kernels + hipBLASLt GEMMs, padded batched attention\"}\n",
-                    tokens, batch, max_q, ms, tokens / (ms * 1e-3), iterations, layer.workspaceBytes(dyn));
+                    "\"attention\": \"%s\", "
+                    "\"note\": \"C++ LlamaContextDecoderLayer: launch* kernels + hipBLASLt GEMMs; attention fused on the matrix cores for fp16 heads of 128 unless ISP_LAYERS_ATTENTION=padded\"}\n",
+                    tokens, batch, max_q, ms, tokens / (ms * 1e-3), iterations, layer.workspaceBytes(dyn), attention_kind());
     } catch (const std::exception& e) {
         std::printf("exception: %s\n", e.what());
         return 1;

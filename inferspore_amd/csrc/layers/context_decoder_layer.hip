@@ -13,6 +13,7 @@
 #include <map>
 #include <string>
 #include <tuple>
+#include <type_traits>
 #include <utility>
 #include <vector>
 #include <algorithm>
@@ -437,6 +438,10 @@ LlamaContextDecoderLayer<T>::LlamaContextDecoderLayer(int head_num, int kv_head_
     LLM_CHECK_WITH_INFO(head_num > 0 && kv_head_num > 0 && head_num % kv_head_num == 0 && head_size > 0 && inter_size > 0,
                         "inconsistent layer dimensions");
     gemm_.reset(new isp_layers::GemmEngine(allocator));
+    const char* attention = std::getenv("ISP_LAYERS_ATTENTION");
+    fused_attention_ = std::is_same<T, half>::value &&
+                       isp_layers::fused_context_attention_supports(head_size, head_num, kv_head_num) &&
+                       !(attention != nullptr && std::strcmp(attention, "padded") == 0);
 }
 
 template <typename T>
@@ -447,9 +452,9 @@ LlamaContextDecoderLayer<T>::~LlamaContextDecoderLayer() {
 template <typename T>
 size_t LlamaContextDecoderLayer<T>::workspaceBytes(const LLaMAAttentionDynParams& d) const {
     const size_t tokens = d.num_tokens, b = d.batch_size, q = d.max_q_len, k = d.max_k_len, hs = head_size_;
-    const size_t elems = tokens * (head_num_ + 2 * kv_head_num_) * hs + b * head_num_ * q * hs +
-                         2 * b * head_num_ * k * hs + b * head_num_ * q * k + b * head_num_ * q * hs +
-                         tokens * head_num_ * hs + tokens * 2 * inter_size_ + tokens * inter_size_;
+    size_t elems = tokens * (head_num_ + 2 * kv_head_num_) * hs + b * head_num_ * q * hs + tokens * head_num_ * hs +
+                   tokens * 2 * inter_size_ + tokens * inter_size_;
+    if (!fused_attention_) elems += 2 * b * head_num_ * k * hs + b * head_num_ * q * k + b * head_num_ * q * hs;
     return elems * sizeof(T);
 }
 
@@ -462,18 +467,22 @@ void LlamaContextDecoderLayer<T>::allocForForward(const LLaMAAttentionDynParams&
     };
     qkv_buf_ = take(tokens * (head_num_ + 2 * kv_head_num_) * hs);
     q_buf_ = take(b * head_num_ * q * hs);
-    k_all_ = take(b * head_num_ * k * hs);
-    v_all_ = take(b * head_num_ * k * hs);
-    scores_ = take(b * head_num_ * q * k);
-    ctx_ = take(b * head_num_ * q * hs);
+    if (!fused_attention_) {
+        k_all_ = take(b * head_num_ * k * hs);
+        v_all_ = take(b * head_num_ * k * hs);
+        scores_ = take(b * head_num_ * q * k);
+        ctx_ = take(b * head_num_ * q * hs);
+    }
     ctx_packed_ = take(tokens * head_num_ * hs);
     gate_up_ = take(tokens * 2 * inter_size_);
     act_ = take(tokens * inter_size_);
     // padded positions of q (and the k / v rows past a sequence's context) are never written by the
     // kernels; they only meet zero probabilities or discarded rows, but must not hold NaN patterns
     CHECK(hipMemsetAsync(q_buf_, 0, b * head_num_ * q * hs * sizeof(T), nullptr));
-    CHECK(hipMemsetAsync(k_all_, 0, b * head_num_ * k * hs * sizeof(T), nullptr));
-    CHECK(hipMemsetAsync(v_all_, 0, b * head_num_ * k * hs * sizeof(T), nullptr));
+    if (!fused_attention_) {
+        CHECK(hipMemsetAsync(k_all_, 0, b * head_num_ * k * hs * sizeof(T), nullptr));
+        CHECK(hipMemsetAsync(v_all_, 0, b * head_num_ * k * hs * sizeof(T), nullptr));
+    }
     allocated_ = d;
 }
 
@@ -537,22 +546,36 @@ void LlamaContextDecoderLayer<T>::forward(TensorMap& inputs, LlamaLayerWeight<T>
     TensorWrapper<T> q_t(GPU, dt, {batch, head_num_, max_q, hs}, q_buf_);
     launchAddFusedQKVBiasTransposeRoPEAndConcatKV(&q_t, &qkv_t, attn.qkv, padding_offset, history_length,
                                                   input_length, layer_id, k_cache, v_cache, attn_params_);
-    // 3. cache -> k, v of every query head over the whole context (GQA broadcast)
-    TensorWrapper<T> k_all_t(GPU, dt, {batch, head_num_, max_k, hs}, k_all_);
-    TensorWrapper<T> v_all_t(GPU, dt, {batch, head_num_, max_k, hs}, v_all_);
-    launchRepeatKVCache(k_cache, v_cache, context_length, layer_id, &k_all_t, &v_all_t);
-    // 4. attention: scores = q k^T, masked softmax, ctx = p v   (batched GEMMs, linear.cu:67-109)
-    const int bh = batch * head_num_;
-    gemm_->matmul(lt, q_buf_, k_all_, scores_, max_q, max_k, hs, true, hs, hs, max_k, bh, (long long)max_q * hs,
-                  (long long)max_k * hs, (long long)max_q * max_k);
-    isp_layers::launch_masked_scaled_softmax(scores_, history_length->data, input_length->data, context_length->data,
-                                             batch, head_num_, max_q, max_k, 1.0f / std::sqrt((float)hs));
-    gemm_->matmul(lt, scores_, v_all_, ctx_, max_q, hs, max_k, false, max_k, hs, hs, bh, (long long)max_q * max_k,
-                  (long long)max_k * hs, (long long)max_q * hs);
-    // 5. [batch, heads, max_q, hs] -> packed [tokens, heads, hs]
-    TensorWrapper<T> ctx_t(GPU, dt, {batch, head_num_, max_q, hs}, ctx_);
-    TensorWrapper<T> packed_t(GPU, dt, {tokens, head_num_, hs}, ctx_packed_);
-    launchTransposeOutRemovePadding(&ctx_t, padding_offset, &packed_t);
+    if (fused_attention_) {
+        // 3-5. attention over the cache itself, straight to packed [tokens, heads, hs]: one kernel
+        LLM_CHECK_WITH_INFO(k_cache->shape[2] == kv_head_num_ && k_cache->shape[4] == hs && v_cache->shape == k_cache->shape,
+                            "k / v cache extents should match the layer's");
+        const int layer = layer_id->getVal();
+        LLM_CHECK_WITH_INFO(layer >= 0 && layer < k_cache->shape[0] && k_cache->shape[1] >= batch, "layer id or batch outside the cache");
+        const size_t slice = (size_t)layer * k_cache->shape[1] * k_cache->shape[2] * k_cache->shape[3] * k_cache->shape[4];
+        if constexpr (std::is_same<T, half>::value)
+            isp_layers::launch_fused_context_attention(q_buf_, k_cache->data + slice, v_cache->data + slice, ctx_packed_,
+                                                       history_length->data, input_length->data, context_length->data,
+                                                       batch, head_num_, kv_head_num_, max_q, max_k, k_cache->shape[3],
+                                                       tokens, 1.0f / std::sqrt((float)hs));
+    } else {
+        // 3. cache -> k, v of every query head over the whole context (GQA broadcast)
+        TensorWrapper<T> k_all_t(GPU, dt, {batch, head_num_, max_k, hs}, k_all_);
+        TensorWrapper<T> v_all_t(GPU, dt, {batch, head_num_, max_k, hs}, v_all_);
+        launchRepeatKVCache(k_cache, v_cache, context_length, layer_id, &k_all_t, &v_all_t);
+        // 4. attention: scores = q k^T, masked softmax, ctx = p v   (batched GEMMs, linear.cu:67-109)
+        const int bh = batch * head_num_;
+        gemm_->matmul(lt, q_buf_, k_all_, scores_, max_q, max_k, hs, true, hs, hs, max_k, bh, (long long)max_q * hs,
+                      (long long)max_k * hs, (long long)max_q * max_k);
+        isp_layers::launch_masked_scaled_softmax(scores_, history_length->data, input_length->data, context_length->data,
+                                                 batch, head_num_, max_q, max_k, 1.0f / std::sqrt((float)hs));
+        gemm_->matmul(lt, scores_, v_all_, ctx_, max_q, hs, max_k, false, max_k, hs, hs, bh, (long long)max_q * max_k,
+                      (long long)max_k * hs, (long long)max_q * hs);
+        // 5. [batch, heads, max_q, hs] -> packed [tokens, heads, hs]
+        TensorWrapper<T> ctx_t(GPU, dt, {batch, head_num_, max_q, hs}, ctx_);
+        TensorWrapper<T> packed_t(GPU, dt, {tokens, head_num_, hs}, ctx_packed_);
+        launchTransposeOutRemovePadding(&ctx_t, padding_offset, &packed_t);
+    }
     // 6. output projection into decoder_input's storage (its contents are no longer needed)   (linear.cu:8)
     const bool o_oi = stored_out_in(attn.output, hidden_, hidden_, "attention output");
     gemm_->matmul(lt, ctx_packed_, attn.output.data, decoder_input->data, tokens, hidden_, hidden_, o_oi, hidden_,

@@ -65,12 +65,20 @@ def reference_layer(residual_rows, lens, w, nh, kvh, hs, base=10000.0):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype,tol", [("f32", 2e-4), ("f16", 3e-2)])
-@pytest.mark.parametrize("nh,kvh,hs,inter", [(2, 2, 128, 512), (4, 2, 64, 384)])
-def test_cpp_context_layer_matches_float64(tmp_path, dtype, tol, nh, kvh, hs, inter):
+@pytest.mark.parametrize("nh,kvh,hs,inter,attention", [(2, 2, 128, 512, "fused"), (4, 2, 128, 512, "fused"),
+                                                        (2, 2, 128, 512, "padded"), (4, 2, 64, 384, "fused")])
+def test_cpp_context_layer_matches_float64(tmp_path, dtype, tol, nh, kvh, hs, inter, attention):
+    """fp16 layers with 128-element heads run the fused attention kernel unless the environment asks for the padded
+    batched form; fp32 layers and other head sizes always run the padded form."""
     assert os.path.exists(EXE), "build/bin/test_context_layer is missing: run python -m inferspore_amd.build"
-    print("[case] test_context_layer %s %d/%d heads x %d, inter %d" % (dtype, nh, kvh, hs, inter), flush=True)
+    print("[case] test_context_layer %s %d/%d heads x %d, inter %d, %s attention" % (dtype, nh, kvh, hs, inter, attention),
+          flush=True)
+    env = dict(os.environ)
+    env.pop("ISP_LAYERS_ATTENTION", None)
+    if attention == "padded":
+        env["ISP_LAYERS_ATTENTION"] = "padded"
     p = subprocess.run([EXE, dtype, str(tmp_path), str(nh), str(kvh), str(hs), str(inter)], stdout=subprocess.PIPE,
-                       stderr=subprocess.STDOUT, text=True, timeout=200)
+                       stderr=subprocess.STDOUT, text=True, timeout=200, env=env)
     assert p.returncode == 0 and "passed" in p.stdout, p.stdout[-3000:]
     H, lens, layers, max_seq = nh * hs, [16, 5, 11], 2, 32
     load = lambda name: np.fromfile(os.path.join(str(tmp_path), name + ".bin"), np.float32).astype(np.float64)
@@ -95,6 +103,15 @@ def test_cpp_context_layer_matches_float64(tmp_path, dtype, tol, nh, kvh, hs, in
             err, scale = np.abs(cache[1, b, :, :l] - exp_rows[b]).max(), np.abs(exp_rows[b]).max()
             assert err <= tol * scale, "%s row block %d: max error %g vs scale %g" % (name, b, err, scale)
             assert not cache[1, b, :, l:].any(), "rows past the sequence must stay untouched"
+
+
+@pytest.mark.gpu
+def test_cpp_fused_context_attention_matches_float64():
+    exe = os.path.join(ROOT, "build", "bin", "test_context_attention")
+    assert os.path.exists(exe), "build/bin/test_context_attention is missing: run python -m inferspore_amd.build"
+    print("[case] test_context_attention", flush=True)
+    p = subprocess.run([exe], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=200)
+    assert p.returncode == 0 and "context attention: passed" in p.stdout, p.stdout[-3000:]
 
 
 def test_layers_library_exports_the_layer_classes():
