@@ -16,7 +16,8 @@
 // The B operand's 16 contraction indices are matched to the accumulator rows by reading V^T's keys in the
 // order (4 h + j, 8 + 4 h + j), h = lane / 32: a contraction does not care about the order of its terms as
 // long as both operands agree.  K tiles sit in LDS as stored ([key][d], padded rows), V tiles transposed
-// ([d][key], written two keys at a time) so that the A operand of the second product is two 8-byte reads.
+// ([d][key], written two keys at a time, the keys of a row in the operand's order) so that the A operand of the
+// second product is one 16-byte read.
 #include <hip/hip_fp16.h>
 #include <hip/hip_runtime.h>
 
@@ -42,12 +43,16 @@ constexpr int kQueryTile = kQueriesPerWave * kWaves;  // queries per workgroup
 constexpr int kKeyTile = 64;
 constexpr int kKStride = kHeadSize + 8;  // halfs per key row in LDS: 272 bytes, spreads the rows over the banks
 
-// The transposed value tile: row d holds the tile's 64 keys as 16 groups of 4 keys (8 bytes, what one operand
-// read takes); group p of row d sits at position p ^ ((d / 2) % 16).  With that exchange the 64 lanes of an operand
-// read (32 rows d, two groups) touch every bank equally, and the transposing writes (pairs of keys, 4 bytes) are
-// spread over half of the banks instead of two.
-__device__ __forceinline__ int vt_dword(int d, int key_group, int dword_in_group) {
-    return d * (kKeyTile / 2) + 2 * (key_group ^ ((d >> 1) & 15)) + dword_in_group;
+// The transposed value tile: row d holds the tile's 64 keys as 8 units of 16 bytes, and a unit is exactly what one
+// lane needs for one product: unit 2 t + h holds the keys 16 t + 4 h + 0..3 followed by 16 t + 8 + 4 h + 0..3 (the
+// order in which the accumulator rows of the scores meet the operand's contraction index).  Unit u of row d sits
+// at position u ^ (d % 8) ^ ((d / 8) % 8): the 64 lanes of an operand read (32 rows d, two units) then touch every
+// bank equally, and the transposing writes (two neighbouring keys, 4 bytes) are spread over half of the banks.
+__device__ __forceinline__ int vt_unit(int d, int unit) { return d * (kKeyTile / 2) + 4 * (unit ^ (d & 7) ^ ((d >> 3) & 7)); }
+// dword that holds the keys `pair * 2` and `pair * 2 + 1` of row d
+__device__ __forceinline__ int vt_pair(int d, int pair) {
+    const int key = 2 * pair, step = key / 16, quad = (key % 16) / 4;  // quads 0..3 of a step: h = quad % 2, second half = quad / 2
+    return vt_unit(d, 2 * step + quad % 2) + 2 * (quad / 2) + (key % 4) / 2;
 }
 
 __device__ __forceinline__ int uniform_int(const int* p, int i) {
@@ -68,6 +73,8 @@ __global__ __launch_bounds__(256, 2) void context_attention_f16(
     const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64, half_id = lane / 32, col = lane % 32;
     // grid: x = head (fastest), y = sequence, z = query tile in DESCENDING order -- the tiles far down the causal
     // triangle visit the most key tiles, and workgroups are handed out in grid order, so the long ones start first
+    // (the kernel takes as long as its longest workgroup: pinning the query tiles of a (sequence, head) pair to one
+    // XCD so that they share its L2 gives up that order and measured 50 instead of 41 us)
     const int head = blockIdx.x, b = blockIdx.y, q0 = (int)(gridDim.z - 1 - blockIdx.z) * kQueryTile;
     const int len = min(uniform_int(input_length, b), max_q_len);
     if (q0 >= len) return;  // workgroup-uniform: only padded queries here
@@ -137,17 +144,21 @@ __global__ __launch_bounds__(256, 2) void context_attention_f16(
             uint32_t lo[4], hi[4];
 #pragma unroll
             for (int j = 0; j < 2; j++) {
-                const uint32_t keep = kt + key + j < wg_visible ? 0xffffffffu : 0u;
-                const uint4 kk = make_uint4(kraw[i][j].x & keep, kraw[i][j].y & keep, kraw[i][j].z & keep, kraw[i][j].w & keep);
+                uint4 kk = kraw[i][j], vv = vraw[i][j];
+                if (kt + kKeyTile > wg_visible) {  // workgroup-uniform: only the last tile has rows to blank
+                    const uint32_t keep = kt + key + j < wg_visible ? 0xffffffffu : 0u;
+                    kk = make_uint4(kk.x & keep, kk.y & keep, kk.z & keep, kk.w & keep);
+                    vv = make_uint4(vv.x & keep, vv.y & keep, vv.z & keep, vv.w & keep);
+                }
                 *reinterpret_cast<uint4*>(&k_lds[(key + j) * kKStride + d0]) = kk;
                 uint32_t* v = j == 0 ? lo : hi;
-                v[0] = vraw[i][j].x & keep, v[1] = vraw[i][j].y & keep, v[2] = vraw[i][j].z & keep, v[3] = vraw[i][j].w & keep;
+                v[0] = vv.x, v[1] = vv.y, v[2] = vv.z, v[3] = vv.w;
             }
 #pragma unroll
             for (int e = 0; e < 8; e++) {
-                const uint32_t a = e % 2 ? lo[e / 2] >> 16 : lo[e / 2] & 0xffffu;       // v[key][d0 + e]
-                const uint32_t c = e % 2 ? hi[e / 2] & 0xffff0000u : hi[e / 2] << 16;   // v[key + 1][d0 + e]
-                vt_lds[vt_dword(d0 + e, pair / 2, pair % 2)] = a | c;
+                // low half: v[key][d0 + e], high half: v[key + 1][d0 + e]  (one byte-permute of the two source dwords)
+                vt_lds[vt_pair(d0 + e, pair)] =
+                    __builtin_amdgcn_perm(hi[e / 2], lo[e / 2], e % 2 ? 0x07060302u : 0x05040100u);
             }
         }
         fetch(kt + kKeyTile);  // past the last tile this re-reads the last visible row and is never stored
@@ -155,16 +166,20 @@ __global__ __launch_bounds__(256, 2) void context_attention_f16(
 
         if (kt < wave_visible) {  // wavefront-uniform: tiles behind this wavefront's diagonal are skipped
             // ---- S^T[key, query] for the 64 keys: two 32-row blocks, 8 steps over d each
+            // The operand reads of a block are issued together, ahead of the products that use them: read one at a
+            // time, each would be waited for (an LDS round trip of a hundred cycles and more) before its product.
             float16v s[2];
 #pragma unroll
             for (int rb = 0; rb < 2; rb++) {
 #pragma unroll
                 for (int i = 0; i < 16; i++) s[rb][i] = 0.0f;
+                half8 ka[8];
 #pragma unroll
-                for (int st = 0; st < 8; st++) {
-                    const half8 a = *reinterpret_cast<const half8*>(&k_lds[(32 * rb + col) * kKStride + 16 * st + 8 * half_id]);
-                    s[rb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, qf[st], s[rb], 0, 0, 0);
-                }
+                for (int st = 0; st < 8; st++)
+                    ka[st] = *reinterpret_cast<const half8*>(&k_lds[(32 * rb + col) * kKStride + 16 * st + 8 * half_id]);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int st = 0; st < 8; st++) s[rb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ka[st], qf[st], s[rb], 0, 0, 0);
             }
             // ---- online softmax; accumulator i of block rb is key kt + 32 rb + 8 (i / 4) + 4 half_id + i % 4
             float tile_max = -INFINITY;
@@ -207,17 +222,16 @@ __global__ __launch_bounds__(256, 2) void context_attention_f16(
 #pragma unroll
             for (int t = 0; t < 4; t++) {
                 const int rb = t / 2, g0 = 2 * (t % 2);
+                half8 va[4];
+#pragma unroll
+                for (int db = 0; db < 4; db++)
+                    va[db] = *reinterpret_cast<const half8*>(&vt_lds[vt_unit(32 * db + col, 2 * t + half_id)]);
                 half8 p;
 #pragma unroll
                 for (int e = 0; e < 8; e++) p[e] = (_Float16)s[rb][4 * (g0 + e / 4) + (e % 4)];
+                __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                for (int db = 0; db < 4; db++) {
-                    const int d = 32 * db + col;
-                    const half4 lo = *reinterpret_cast<const half4*>(&vt_lds[vt_dword(d, 4 * t + half_id, 0)]);
-                    const half4 hi = *reinterpret_cast<const half4*>(&vt_lds[vt_dword(d, 4 * t + half_id + 2, 0)]);
-                    const half8 a = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-                    acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, p, acc[db], 0, 0, 0);
-                }
+                for (int db = 0; db < 4; db++) acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(va[db], p, acc[db], 0, 0, 0);
             }
         }
         __syncthreads();  // the next tile overwrites LDS
