@@ -23,7 +23,7 @@
 // two batched attention GEMMs are hipBLASLt calls made here; the softmax between them is a kernel of
 // the layers library's own.  That padded, batched attention is the reference's own design
 // (src/kernels/linear.cu:67-109, attn_softmax_kernel.cu:50-125) and what fp32 layers and head sizes other
-// than 128 run.  For fp16 heads of 128 elements the three attention lines (KV broadcast, the two batched
+// than 128 and 64 run.  For fp16 heads of 128 or 64 elements the three attention lines (KV broadcast, the two batched
 // GEMMs with the softmax, the transpose) are replaced by ONE fused kernel on the matrix cores that reads
 // the cache directly and writes the packed rows (launch_fused_context_attention below);
 // ISP_LAYERS_ATTENTION=padded in the environment keeps the padded form.
@@ -59,18 +59,18 @@ void launch_masked_scaled_softmax(T* scores, const int* history_length, const in
                                   const int* context_length, int batch, int head_num, int max_q_len,
                                   int max_k_len, float scale);
 
-// The fused causal attention for fp16 heads of 128 elements (one kernel on the matrix cores in place of KV
+// The fused causal attention for fp16 heads of hs = 128 or 64 elements (one kernel on the matrix cores in place of KV
 // broadcast, q x k^T, the softmax above, p x v and the transpose back to packed tokens; null stream):
-//   q_buf            [batch, head_num, max_q_len, 128], rows of padded queries are never read
-//   k_cache, v_cache the layer's slice [batch, kv_head_num, max_seq_len, 128] holding history and current keys
-//   out              [tokens, head_num, 128], row (first token of b) + q for every q < input_length[b]
+//   q_buf            [batch, head_num, max_q_len, hs], rows of padded queries are never read
+//   k_cache, v_cache the layer's slice [batch, kv_head_num, max_seq_len, hs] holding history and current keys
+//   out              [tokens, head_num, hs], row (first token of b) + q for every q < input_length[b]
 // with the same visibility rule as the softmax.  fused_context_attention_supports() says whether a layer
 // of these dimensions can use it.
 bool fused_context_attention_supports(int head_size, int head_num, int kv_head_num);
 void launch_fused_context_attention(const half* q_buf, const half* k_cache, const half* v_cache, half* out,
                                     const int* history_length, const int* input_length, const int* context_length,
-                                    int batch, int head_num, int kv_head_num, int max_q_len, int max_k_len,
-                                    int max_seq_len, int tokens, float scale);
+                                    int batch, int head_num, int kv_head_num, int head_size, int max_q_len,
+                                    int max_k_len, int max_seq_len, int tokens, float scale);
 }
 
 template <typename T>
@@ -100,7 +100,7 @@ private:
     float eps_;
     BaseAllocator* allocator_;
     std::unique_ptr<isp_layers::GemmEngine> gemm_;
-    bool fused_attention_ = false;  // fp16 heads of 128: the fused kernel instead of steps 3-5 of the padded form
+    bool fused_attention_ = false;  // fp16 heads of 128 or 64: the fused kernel instead of steps 3-5 of the padded form
 
     LLaMAAttentionDynParams allocated_;
     T* qkv_buf_ = nullptr;      // [tokens, head_num + 2 kv_head_num, head_size]

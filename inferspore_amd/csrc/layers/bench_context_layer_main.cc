@@ -94,7 +94,7 @@ int main(int argc, char** argv) {
                     "\"max_q_len\": %d, \"ms_per_layer\": %.6f, \"tokens_per_s_per_layer\": %.1f, \"iterations\": %d, "
                     "\"activation_buffer_bytes\": %zu, "
                     "\"attention\": \"%s\", "
-                    "\"note\": \"C++ LlamaContextDecoderLayer: launch* kernels + hipBLASLt GEMMs; attention fused on the matrix cores for fp16 heads of 128 unless ISP_LAYERS_ATTENTION=padded\"}\n",
+                    "\"note\": \"C++ LlamaContextDecoderLayer: launch* kernels + hipBLASLt GEMMs; attention fused on the matrix cores for fp16 heads of 128 or 64 unless ISP_LAYERS_ATTENTION=padded\"}\n",
                     tokens, batch, max_q, ms, tokens / (ms * 1e-3), iterations, layer.workspaceBytes(dyn), attention_kind());
     } catch (const std::exception& e) {
         std::printf("exception: %s\n", e.what());

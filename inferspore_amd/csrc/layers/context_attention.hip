@@ -1,8 +1,8 @@
-// Fused causal attention of the context-decoder layer for fp16 heads of 128 elements: one kernel in place of
+// Fused causal attention of the context-decoder layer for fp16 heads of 128 or 64 elements: one kernel in place of
 // KV broadcast, q x k^T, masked softmax, p x v and the transpose back to packed tokens.  It reads the padded
-// queries [batch, head_num, max_q_len, 128], the layer's slice of the KV cache [batch, kv_head_num,
-// max_seq_len, 128] (keys and values of the history and of this call's tokens) and writes the packed
-// [tokens, head_num, 128] rows the output projection consumes.  The [queries x keys] scores never leave the
+// queries [batch, head_num, max_q_len, hs], the layer's slice of the KV cache [batch, kv_head_num,
+// max_seq_len, hs] (keys and values of the history and of this call's tokens) and writes the packed
+// [tokens, head_num, hs] rows the output projection consumes.  The [queries x keys] scores never leave the
 // registers, and key tiles behind the causal diagonal are not visited.
 //
 // The mask is the one of the layer's softmax: query q of sequence b sees the keys at positions
@@ -36,12 +36,11 @@ typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef _Float16 half4 __attribute__((ext_vector_type(4)));
 typedef float float16v __attribute__((ext_vector_type(16)));
 
-constexpr int kHeadSize = 128;
 constexpr int kQueriesPerWave = 32;
 constexpr int kWaves = 4;
 constexpr int kQueryTile = kQueriesPerWave * kWaves;  // queries per workgroup
 constexpr int kKeyTile = 64;
-constexpr int kKStride = kHeadSize + 8;  // halfs per key row in LDS: 272 bytes, spreads the rows over the banks
+constexpr int kKPad = 8;  // halfs added to a key row in LDS (272 bytes for 128-element heads): spreads the rows over the banks
 
 // The transposed value tile: row d holds the tile's 64 keys as 8 units of 16 bytes, and a unit is exactly what one
 // lane needs for one product: unit 2 t + h holds the keys 16 t + 4 h + 0..3 followed by 16 t + 8 + 4 h + 0..3 (the
@@ -63,10 +62,16 @@ __device__ __forceinline__ int uniform_int(const int* p, int i) {
 
 __device__ __forceinline__ float other_half(float x) { return __shfl_xor(x, 32, 64); }
 
+template <int HS>  // head size: 128 or 64
 __global__ __launch_bounds__(256, 2) void context_attention_f16(
     const _Float16* __restrict__ q_buf, const _Float16* __restrict__ k_cache, const _Float16* __restrict__ v_cache,
     _Float16* __restrict__ out, const int* history_length, const int* input_length, const int* context_length,
     int head_num, int kv_head_num, int max_q_len, int max_k_len, int max_seq_len, int tokens, float scale_log2e) {
+    constexpr int kHeadSize = HS, kKStride = HS + kKPad;
+    constexpr int kDSteps = HS / 16;    // products over d per 32 x 32 block of scores
+    constexpr int kDBlocks = HS / 32;   // 32-row blocks of O^T
+    constexpr int kChunks = HS / 8;     // 16-byte pieces of a key or value row
+    constexpr int kMoves = HS / 64;     // key pairs a thread moves per tile
     __shared__ __align__(16) _Float16 k_lds[kKeyTile * kKStride];
     __shared__ __align__(16) uint32_t vt_lds[kHeadSize * kKeyTile / 2];  // [d][key], two keys per dword
 
@@ -98,19 +103,19 @@ __global__ __launch_bounds__(256, 2) void context_attention_f16(
     const int my_visible = real ? min(hist + my_q + 1, ctx) : 0;
 
     // Q^T as the B operand: lane (col, half_id) holds q[my_q][16 s + 8 half_id + 0..7] for the 8 steps over d
-    half8 qf[8];
+    half8 qf[kDSteps];
     {
         const _Float16* q_row = q_buf + (((size_t)b * head_num + head) * (size_t)max_q_len + (size_t)(real ? my_q : q0)) * kHeadSize;
 #pragma unroll
-        for (int s = 0; s < 8; s++) {
+        for (int s = 0; s < kDSteps; s++) {
             qf[s] = *reinterpret_cast<const half8*>(q_row + 16 * s + 8 * half_id);
             if (!real) qf[s] = half8{0, 0, 0, 0, 0, 0, 0, 0};
         }
     }
 
-    float16v acc[4];  // O^T[d = 32 db + rows, query = col]
+    float16v acc[kDBlocks];  // O^T[d = 32 db + rows, query = col]
 #pragma unroll
-    for (int db = 0; db < 4; db++)
+    for (int db = 0; db < kDBlocks; db++)
 #pragma unroll
         for (int i = 0; i < 16; i++) acc[db][i] = 0.0f;
     float run_max = -INFINITY, run_sum = 0.0f;
@@ -120,11 +125,11 @@ __global__ __launch_bounds__(256, 2) void context_attention_f16(
     // re-reads the last visible one and is masked to zero when it is stored (loads or register writes under a
     // branch would each be waited for before the next is issued).  The loads of tile n + 1 are in flight while
     // tile n is computed.
-    uint4 kraw[2][2], vraw[2][2];
+    uint4 kraw[kMoves][2], vraw[kMoves][2];
     auto fetch = [&](int kt) {
 #pragma unroll
-        for (int i = 0; i < 2; i++) {
-            const int unit = tid + 256 * i, d0 = (unit % 16) * 8, key = 2 * (unit / 16);
+        for (int i = 0; i < kMoves; i++) {
+            const int unit = tid + 256 * i, d0 = (unit % kChunks) * 8, key = 2 * (unit / kChunks);
 #pragma unroll
             for (int j = 0; j < 2; j++) {
                 const size_t at = (size_t)min(kt + key + j, wg_visible - 1) * kHeadSize + d0;
@@ -139,8 +144,8 @@ __global__ __launch_bounds__(256, 2) void context_attention_f16(
         // ---- the tile into LDS: 64 keys x 128 d of K as stored, of V transposed; keys past the visible ones as zeros
         //      (a zero probability times whatever an unwritten cache row holds could be NaN)
 #pragma unroll
-        for (int i = 0; i < 2; i++) {
-            const int unit = tid + 256 * i, pair = unit / 16, d0 = (unit % 16) * 8, key = 2 * pair;
+        for (int i = 0; i < kMoves; i++) {
+            const int unit = tid + 256 * i, pair = unit / kChunks, d0 = (unit % kChunks) * 8, key = 2 * pair;
             uint32_t lo[4], hi[4];
 #pragma unroll
             for (int j = 0; j < 2; j++) {
@@ -173,13 +178,13 @@ __global__ __launch_bounds__(256, 2) void context_attention_f16(
             for (int rb = 0; rb < 2; rb++) {
 #pragma unroll
                 for (int i = 0; i < 16; i++) s[rb][i] = 0.0f;
-                half8 ka[8];
+                half8 ka[kDSteps];
 #pragma unroll
-                for (int st = 0; st < 8; st++)
+                for (int st = 0; st < kDSteps; st++)
                     ka[st] = *reinterpret_cast<const half8*>(&k_lds[(32 * rb + col) * kKStride + 16 * st + 8 * half_id]);
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                for (int st = 0; st < 8; st++) s[rb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ka[st], qf[st], s[rb], 0, 0, 0);
+                for (int st = 0; st < kDSteps; st++) s[rb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ka[st], qf[st], s[rb], 0, 0, 0);
             }
             // ---- online softmax; accumulator i of block rb is key kt + 32 rb + 8 (i / 4) + 4 half_id + i % 4
             float tile_max = -INFINITY;
@@ -214,7 +219,7 @@ __global__ __launch_bounds__(256, 2) void context_attention_f16(
             run_max = new_max;
             if (__any(rescale != 1.0f)) {  // the running maximum moves in the first tiles and rarely afterwards
 #pragma unroll
-                for (int db = 0; db < 4; db++)
+                for (int db = 0; db < kDBlocks; db++)
 #pragma unroll
                     for (int i = 0; i < 16; i++) acc[db][i] *= rescale;
             }
@@ -222,16 +227,16 @@ __global__ __launch_bounds__(256, 2) void context_attention_f16(
 #pragma unroll
             for (int t = 0; t < 4; t++) {
                 const int rb = t / 2, g0 = 2 * (t % 2);
-                half8 va[4];
+                half8 va[kDBlocks];
 #pragma unroll
-                for (int db = 0; db < 4; db++)
+                for (int db = 0; db < kDBlocks; db++)
                     va[db] = *reinterpret_cast<const half8*>(&vt_lds[vt_unit(32 * db + col, 2 * t + half_id)]);
                 half8 p;
 #pragma unroll
                 for (int e = 0; e < 8; e++) p[e] = (_Float16)s[rb][4 * (g0 + e / 4) + (e % 4)];
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                for (int db = 0; db < 4; db++) acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(va[db], p, acc[db], 0, 0, 0);
+                for (int db = 0; db < kDBlocks; db++) acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(va[db], p, acc[db], 0, 0, 0);
             }
         }
         __syncthreads();  // the next tile overwrites LDS
@@ -243,7 +248,7 @@ __global__ __launch_bounds__(256, 2) void context_attention_f16(
         const float inv = run_sum > 0.0f ? 1.0f / run_sum : 0.0f;
         _Float16* o_row = out + ((size_t)token * head_num + head) * kHeadSize;
 #pragma unroll
-        for (int db = 0; db < 4; db++)
+        for (int db = 0; db < kDBlocks; db++)
 #pragma unroll
             for (int g = 0; g < 4; g++) {
                 half4 v;
@@ -257,15 +262,16 @@ __global__ __launch_bounds__(256, 2) void context_attention_f16(
 }  // namespace
 
 bool fused_context_attention_supports(int head_size, int head_num, int kv_head_num) {
-    return head_size == kHeadSize && kv_head_num > 0 && head_num % kv_head_num == 0 && head_num <= 65535;
+    return (head_size == 128 || head_size == 64) && kv_head_num > 0 && head_num % kv_head_num == 0;
 }
 
 void launch_fused_context_attention(const half* q_buf, const half* k_cache, const half* v_cache, half* out,
                                     const int* history_length, const int* input_length, const int* context_length,
-                                    int batch, int head_num, int kv_head_num, int max_q_len, int max_k_len,
-                                    int max_seq_len, int tokens, float scale) {
+                                    int batch, int head_num, int kv_head_num, int head_size, int max_q_len,
+                                    int max_k_len, int max_seq_len, int tokens, float scale) {
     LLM_CHECK_WITH_INFO(q_buf && k_cache && v_cache && out && history_length && input_length && context_length,
                         "fused attention: null operand");
+    LLM_CHECK_WITH_INFO(head_size == 128 || head_size == 64, "fused attention: heads of 128 or 64 elements only");
     LLM_CHECK_WITH_INFO(batch > 0 && batch <= 65535 && head_num > 0 && kv_head_num > 0 && head_num % kv_head_num == 0 &&
                             max_q_len > 0 && (max_q_len + kQueryTile - 1) / kQueryTile <= 65535 && max_k_len > 0 && max_seq_len > 0 &&
                             tokens >= 0 && scale > 0.0f,
@@ -274,10 +280,15 @@ void launch_fused_context_attention(const half* q_buf, const half* k_cache, cons
                            reinterpret_cast<uintptr_t>(v_cache) | reinterpret_cast<uintptr_t>(out);
     LLM_CHECK_WITH_INFO((bits & 15u) == 0, "fused attention: operands must be 16-byte aligned");
     const dim3 grid((unsigned)head_num, (unsigned)batch, (unsigned)((max_q_len + kQueryTile - 1) / kQueryTile));
-    hipLaunchKernelGGL(context_attention_f16, grid, dim3(256), 0, nullptr, reinterpret_cast<const _Float16*>(q_buf),
-                       reinterpret_cast<const _Float16*>(k_cache), reinterpret_cast<const _Float16*>(v_cache),
-                       reinterpret_cast<_Float16*>(out), history_length, input_length, context_length, head_num,
-                       kv_head_num, max_q_len, max_k_len, max_seq_len, tokens, scale * 1.4426950408889634f);
+#define ISP_LAUNCH_ATTENTION(HS)                                                                                  \
+    hipLaunchKernelGGL(context_attention_f16<HS>, grid, dim3(256), 0, nullptr,                                    \
+                       reinterpret_cast<const _Float16*>(q_buf), reinterpret_cast<const _Float16*>(k_cache),      \
+                       reinterpret_cast<const _Float16*>(v_cache), reinterpret_cast<_Float16*>(out), history_length, \
+                       input_length, context_length, head_num, kv_head_num, max_q_len, max_k_len, max_seq_len,   \
+                       tokens, scale * 1.4426950408889634f)
+    if (head_size == 128) ISP_LAUNCH_ATTENTION(128);
+    else ISP_LAUNCH_ATTENTION(64);
+#undef ISP_LAUNCH_ATTENTION
     CHECK(hipGetLastError());
 }
 

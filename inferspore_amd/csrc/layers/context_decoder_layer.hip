@@ -556,7 +556,7 @@ void LlamaContextDecoderLayer<T>::forward(TensorMap& inputs, LlamaLayerWeight<T>
         if constexpr (std::is_same<T, half>::value)
             isp_layers::launch_fused_context_attention(q_buf_, k_cache->data + slice, v_cache->data + slice, ctx_packed_,
                                                        history_length->data, input_length->data, context_length->data,
-                                                       batch, head_num_, kv_head_num_, max_q, max_k, k_cache->shape[3],
+                                                       batch, head_num_, kv_head_num_, hs, max_q, max_k, k_cache->shape[3],
                                                        tokens, 1.0f / std::sqrt((float)hs));
     } else {
         // 3. cache -> k, v of every query head over the whole context (GQA broadcast)

@@ -14,14 +14,14 @@
 
 struct Case {
     const char* name;
-    int head_num, kv_head_num, max_q, max_seq;
+    int head_size, head_num, kv_head_num, max_q, max_seq;
     std::vector<int> lens, hist, ctx_cut;  // ctx = hist + len - ctx_cut
     int max_k_slack;                       // max_k_len = max(ctx) - slack: a max_k_len that cuts the longest context
 };
 
 static void run(const Case& c, std::mt19937& gen) {
     using S = uint16_t;
-    const int hs = 128, batch = (int)c.lens.size();
+    const int hs = c.head_size, batch = (int)c.lens.size();
     std::vector<int> ctx(batch);
     int max_k = 1;
     for (int b = 0; b < batch; b++) {
@@ -53,7 +53,7 @@ static void run(const Case& c, std::mt19937& gen) {
     int *dh = to_device(c.hist), *dl = to_device(c.lens), *dc = to_device(ctx);
     const float scale = 1.0f / std::sqrt((float)hs);
     isp_layers::launch_fused_context_attention((const half*)dq, (const half*)dk, (const half*)dv, (half*)dout, dh, dl, dc,
-                                               batch, c.head_num, c.kv_head_num, c.max_q, max_k, c.max_seq, tokens, scale);
+                                               batch, c.head_num, c.kv_head_num, hs, c.max_q, max_k, c.max_seq, tokens, scale);
     CHECK(hipDeviceSynchronize());
     auto got = to_host(dout, out.size());
 
@@ -94,28 +94,34 @@ static void run(const Case& c, std::mt19937& gen) {
     // keys) and the result once more: 2e-3 of the largest output is several times that
     EXPECT(not_finite == 0, "%s: %lld outputs are NaN or infinite (a row skipped, or unwritten memory read)", c.name, not_finite);
     EXPECT(worst <= 2e-3 * peak, "%s: error %g against a largest output of %g", c.name, worst, peak);
-    std::printf("%-44s %d tokens, max_k %d: error %.2e of peak %.2f\n", c.name, tokens, max_k, worst, peak);
+    std::printf("%-44s heads of %3d, %d tokens, max_k %d: error %.2e of peak %.2f\n", c.name, hs, tokens, max_k, worst, peak);
     for (void* ptr : {(void*)dq, (void*)dk, (void*)dv, (void*)dout, (void*)dh, (void*)dl, (void*)dc}) CHECK(hipFree(ptr));
 }
 
 int main() {
     std::mt19937 gen(20240611);
     const Case cases[] = {
-        {"one short sequence", 2, 2, 5, 8, {5}, {0}, {0}, 0},
-        {"ragged batch with history, grouped heads", 4, 2, 16, 48, {16, 5, 11}, {0, 9, 30}, {0, 0, 0}, 0},
-        {"a context cut short and a max_k_len below it", 4, 4, 16, 48, {16, 7}, {3, 20}, {0, 2}, 1},
-        {"two query tiles, the second partly filled", 2, 2, 200, 300, {200, 133}, {0, 70}, {0, 0}, 0},
-        {"one key head shared by eight query heads", 8, 1, 130, 130, {129}, {0}, {0}, 0},
-        {"a single query over a long history", 4, 2, 1, 1100, {1, 1, 1}, {1000, 63, 64}, {0, 0, 0}, 0},
-        {"keys ending exactly at a tile boundary", 2, 1, 64, 128, {64, 64}, {0, 64}, {0, 0}, 0},
-        {"an empty sequence inside the batch", 2, 2, 40, 64, {40, 0, 17}, {0, 5, 9}, {0, 0, 0}, 0},
+        {"one short sequence", 128, 2, 2, 5, 8, {5}, {0}, {0}, 0},
+        {"ragged batch with history, grouped heads", 128, 4, 2, 16, 48, {16, 5, 11}, {0, 9, 30}, {0, 0, 0}, 0},
+        {"a context cut short and a max_k_len below it", 128, 4, 4, 16, 48, {16, 7}, {3, 20}, {0, 2}, 1},
+        {"two query tiles, the second partly filled", 128, 2, 2, 200, 300, {200, 133}, {0, 70}, {0, 0}, 0},
+        {"one key head shared by eight query heads", 128, 8, 1, 130, 130, {129}, {0}, {0}, 0},
+        {"a single query over a long history", 128, 4, 2, 1, 1100, {1, 1, 1}, {1000, 63, 64}, {0, 0, 0}, 0},
+        {"keys ending exactly at a tile boundary", 128, 2, 1, 64, 128, {64, 64}, {0, 64}, {0, 0}, 0},
+        {"an empty sequence inside the batch", 128, 2, 2, 40, 64, {40, 0, 17}, {0, 5, 9}, {0, 0, 0}, 0},
     };
     try {
-        if (!isp_layers::fused_context_attention_supports(128, 32, 8) || isp_layers::fused_context_attention_supports(64, 32, 8)) {
+        if (!isp_layers::fused_context_attention_supports(128, 32, 8) || !isp_layers::fused_context_attention_supports(64, 32, 8) ||
+            isp_layers::fused_context_attention_supports(96, 32, 8) || isp_layers::fused_context_attention_supports(128, 32, 5)) {
             std::printf("FAIL: fused_context_attention_supports\n");
             g_failures++;
         }
-        for (const Case& c : cases) run(c, gen);
+        for (const Case& c : cases) {
+            run(c, gen);
+            Case narrow = c;  // the same case on 64-element heads
+            narrow.head_size = 64;
+            run(narrow, gen);
+        }
     } catch (const std::exception& e) {
         std::printf("exception: %s\n", e.what());
         return 1;

@@ -66,9 +66,9 @@ def reference_layer(residual_rows, lens, w, nh, kvh, hs, base=10000.0):
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype,tol", [("f32", 2e-4), ("f16", 3e-2)])
 @pytest.mark.parametrize("nh,kvh,hs,inter,attention", [(2, 2, 128, 512, "fused"), (4, 2, 128, 512, "fused"),
-                                                        (2, 2, 128, 512, "padded"), (4, 2, 64, 384, "fused")])
+                                                        (2, 2, 128, 512, "padded"), (4, 2, 64, 384, "fused"), (4, 2, 64, 384, "padded")])
 def test_cpp_context_layer_matches_float64(tmp_path, dtype, tol, nh, kvh, hs, inter, attention):
-    """fp16 layers with 128-element heads run the fused attention kernel unless the environment asks for the padded
+    """fp16 layers with 128- or 64-element heads run the fused attention kernel unless the environment asks for the padded
     batched form; fp32 layers and other head sizes always run the padded form."""
     assert os.path.exists(EXE), "build/bin/test_context_layer is missing: run python -m inferspore_amd.build"
     print("[case] test_context_layer %s %d/%d heads x %d, inter %d, %s attention" % (dtype, nh, kvh, hs, inter, attention),
