@@ -123,3 +123,5 @@ def test_layers_library_exports_the_layer_classes():
         assert "LlamaContextDecoderLayer<%s>::allocForForward(" % t in syms
         assert "LlamaLayerWeight<%s>::loadWeights()" % t in syms
         assert "isp_layers::launch_masked_scaled_softmax<%s>(" % t in syms
+    assert "isp_layers::launch_fused_context_attention(" in syms
+    assert "isp_layers::fused_context_attention_supports(" in syms
