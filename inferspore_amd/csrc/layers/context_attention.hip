@@ -102,6 +102,15 @@ __global__ __launch_bounds__(256, 2) void context_attention_f16(
     const bool real = my_q < len;
     const int my_visible = real ? min(hist + my_q + 1, ctx) : 0;
 
+    const long long token = (long long)first_token + my_q;
+    if (wg_visible <= 0) {  // workgroup-uniform: a context of no keys (inconsistent lengths); nothing to attend to
+        if (real && token < tokens) {
+            _Float16* o_row = out + ((size_t)token * head_num + head) * kHeadSize;
+            for (int d = 8 * half_id; d < kHeadSize; d += 16) *reinterpret_cast<uint4*>(o_row + d) = make_uint4(0u, 0u, 0u, 0u);
+        }
+        return;
+    }
+
     // Q^T as the B operand: lane (col, half_id) holds q[my_q][16 s + 8 half_id + 0..7] for the 8 steps over d
     half8 qf[kDSteps];
     {
@@ -243,7 +252,6 @@ __global__ __launch_bounds__(256, 2) void context_attention_f16(
     }
 
     // ---- O^T / sum -> the packed token row; accumulator i of block db is d = 32 db + 8 (i / 4) + 4 half_id + i % 4
-    const long long token = (long long)first_token + my_q;
     if (real && token < tokens) {
         const float inv = run_sum > 0.0f ? 1.0f / run_sum : 0.0f;
         _Float16* o_row = out + ((size_t)token * head_num + head) * kHeadSize;

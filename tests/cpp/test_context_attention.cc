@@ -109,6 +109,7 @@ int main() {
         {"a single query over a long history", 128, 4, 2, 1, 1100, {1, 1, 1}, {1000, 63, 64}, {0, 0, 0}, 0},
         {"keys ending exactly at a tile boundary", 128, 2, 1, 64, 128, {64, 64}, {0, 64}, {0, 0}, 0},
         {"an empty sequence inside the batch", 128, 2, 2, 40, 64, {40, 0, 17}, {0, 5, 9}, {0, 0, 0}, 0},
+        {"a context of no keys (rows of zeros)", 128, 2, 2, 8, 16, {5, 8}, {0, 0}, {5, 0}, 0},
     };
     try {
         if (!isp_layers::fused_context_attention_supports(128, 32, 8) || !isp_layers::fused_context_attention_supports(64, 32, 8) ||
