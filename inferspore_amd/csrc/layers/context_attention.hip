@@ -72,8 +72,8 @@ __global__ __launch_bounds__(256, 2) void context_attention_f16(
     constexpr int kDBlocks = HS / 32;   // 32-row blocks of O^T
     constexpr int kChunks = HS / 8;     // 16-byte pieces of a key or value row
     constexpr int kMoves = HS / 64;     // key pairs a thread moves per tile
-    __shared__ __align__(16) _Float16 k_lds[kKeyTile * kKStride];
-    __shared__ __align__(16) uint32_t vt_lds[kHeadSize * kKeyTile / 2];  // [d][key], two keys per dword
+    __shared__ __align__(16) _Float16 k_tiles[2][kKeyTile * kKStride];
+    __shared__ __align__(16) uint32_t vt_tiles[2][kHeadSize * kKeyTile / 2];  // [d][key], two keys per dword
 
     const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64, half_id = lane / 32, col = lane % 32;
     // grid: x = head (fastest), y = sequence, z = query tile in DESCENDING order -- the tiles far down the causal
@@ -147,9 +147,9 @@ __global__ __launch_bounds__(256, 2) void context_attention_f16(
             }
         }
     };
-    fetch(0);
-
-    for (int kt = 0; kt < wg_visible; kt += kKeyTile) {
+    auto store = [&](int buf, int kt) {
+        _Float16* k_lds = k_tiles[buf];
+        uint32_t* vt_lds = vt_tiles[buf];
         // ---- the tile into LDS: 64 keys x 128 d of K as stored, of V transposed; keys past the visible ones as zeros
         //      (a zero probability times whatever an unwritten cache row holds could be NaN)
 #pragma unroll
@@ -175,8 +175,16 @@ __global__ __launch_bounds__(256, 2) void context_attention_f16(
                     __builtin_amdgcn_perm(hi[e / 2], lo[e / 2], e % 2 ? 0x07060302u : 0x05040100u);
             }
         }
-        fetch(kt + kKeyTile);  // past the last tile this re-reads the last visible row and is never stored
-        __syncthreads();
+    };
+    fetch(0);
+    store(0, 0);
+    fetch(kKeyTile);  // past the last tile a fetch re-reads the last visible row; what it brings is stored as zeros
+    __syncthreads();
+
+    int cur = 0;
+    for (int kt = 0; kt < wg_visible; kt += kKeyTile, cur ^= 1) {
+        const _Float16* k_lds = k_tiles[cur];
+        const uint32_t* vt_lds = vt_tiles[cur];
 
         if (kt < wave_visible) {  // wavefront-uniform: tiles behind this wavefront's diagonal are skipped
             // ---- S^T[key, query] for the 64 keys: two 32-row blocks, 8 steps over d each
@@ -248,7 +256,12 @@ __global__ __launch_bounds__(256, 2) void context_attention_f16(
                 for (int db = 0; db < kDBlocks; db++) acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(va[db], p, acc[db], 0, 0, 0);
             }
         }
-        __syncthreads();  // the next tile overwrites LDS
+        // the next tile (its loads were issued before this tile's products) goes into the other buffer, which every
+        // wavefront finished reading before the barrier that ended the previous iteration; then the loads of the
+        // tile after it are started: one barrier per tile, and no load is waited for right after it was issued
+        store(cur ^ 1, kt + kKeyTile);
+        fetch(kt + 2 * kKeyTile);
+        __syncthreads();
     }
 
     // ---- O^T / sum -> the packed token row; accumulator i of block db is d = 32 db + 8 (i / 4) + 4 half_id + i % 4
