@@ -60,7 +60,16 @@ __device__ __forceinline__ int uniform_int(const int* p, int i) {
     return reinterpret_cast<constant_ints>((unsigned long long)p)[i];
 }
 
-__device__ __forceinline__ float other_half(float x) { return __shfl_xor(x, 32, 64); }
+// Maximum / sum of a value with the one in the other half of the wavefront (lane ^ 32), without a trip through LDS:
+// the swap leaves the lower half's value in every lane of one register and the upper half's in the other.
+__device__ __forceinline__ float halves_max(float x) {
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float halves_sum(float x) {
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
 
 template <int HS>  // head size: 128 or 64
 __global__ __launch_bounds__(256, 2) void context_attention_f16(
@@ -218,7 +227,7 @@ __global__ __launch_bounds__(256, 2) void context_attention_f16(
             for (int rb = 0; rb < 2; rb++)
 #pragma unroll
                 for (int i = 0; i < 16; i++) tile_max = fmaxf(tile_max, s[rb][i]);
-            tile_max = fmaxf(tile_max, other_half(tile_max));
+            tile_max = halves_max(tile_max);
             const float new_max = fmaxf(run_max, tile_max);
             const float safe_max = new_max == -INFINITY ? 0.0f : new_max;  // a query with no visible key yet
             const float rescale = __builtin_amdgcn_exp2f((run_max - safe_max) * scale_log2e);
@@ -231,7 +240,7 @@ __global__ __launch_bounds__(256, 2) void context_attention_f16(
                     s[rb][i] = __builtin_amdgcn_exp2f(fmaf(s[rb][i], scale_log2e, -mc));
                     tile_sum += s[rb][i];
                 }
-            tile_sum += other_half(tile_sum);
+            tile_sum = halves_sum(tile_sum);
             run_sum = run_sum * rescale + tile_sum;
             run_max = new_max;
             if (__any(rescale != 1.0f)) {  // the running maximum moves in the first tiles and rarely afterwards
