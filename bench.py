@@ -482,20 +482,23 @@ def context_layer_record(torch, steps, warmup, stream):
             "note": "library kernels via the C ABI; GEMMs and attention are torch library calls"}
 
 
-def context_layer_cpp_record(torch, steps, warmup, layers=0, decode=False):
+def context_layer_cpp_record(torch, steps, warmup, layers=0, decode=False, attention=False):
     """The same layer through the C++ layer class (launch* kernels + hipBLASLt GEMMs called directly, attention fused
     on the matrix cores): runs build/bin/bench_context_layer in a child process and returns its JSON record.
     With `layers` > 0: the whole stack of that many layers (LlamaContextDecoder, build/bin/bench_context_decoder).
     With `decode`: one new token for each of 16 sequences that already hold 1023 tokens in the KV cache -- the same
-    layer call as a decode step."""
+    layer call as a decode step.  With `attention`: the layer's fused attention kernel alone (build/bin/bench_context_attention),
+    with its rate against the fp16 MFMA peak over the causal flops."""
     import subprocess
-    name = "bench_context_decoder" if layers else "bench_context_layer"
+    name = "bench_context_attention" if attention else "bench_context_decoder" if layers else "bench_context_layer"
     exe = os.path.join(ROOT, "build", "bin", name)
     if not os.path.exists(exe):
         return {"error": "build/bin/%s is missing (python -m inferspore_amd.build)" % name}
     lens = [str(int(v)) for v in bench_lengths(torch).tolist()]
     counts = [str(layers), "5", "2"] if layers else [str(max(10, steps // 10)), str(max(3, warmup // 4))]
     args = counts + ["512"] + lens
+    if attention:
+        args = [str(max(50, steps // 2)), "10", "512"] + lens
     if decode:
         args = ["--history", "1023", str(max(50, steps // 2)), "10", "1"] + ["1"] * 16
     try:
@@ -858,6 +861,7 @@ def main():
         config["context_layer_cpp"] = context_layer_cpp_record(torch, a.steps, a.warmup)
         config["context_decoder_cpp"] = context_layer_cpp_record(torch, a.steps, a.warmup, layers=32)
         config["context_layer_cpp_decode_step"] = context_layer_cpp_record(torch, a.steps, a.warmup, decode=True)
+        config["context_attention_cpp"] = context_layer_cpp_record(torch, a.steps, a.warmup, attention=True)
         config["decode_sequence"] = decode_sequence_record(torch, stream)
     if not a.kernels_only:
         # cache-resident rates (one buffer set, no rotation): the hot-path configurations by default, every
