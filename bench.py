@@ -12,12 +12,16 @@ Method
   * every launch works on the next of R buffer sets, R chosen so the sets together exceed 1 GiB:
     successive launches cannot be served from the 256 MB last-level cache ("cold"; --warm disables
     the rotation and is reported separately, never as `value`);
-  * after W warm-up launches and a synchronize, a few untimed lead-in launches keep the queue busy and
-    then several regions of exactly K launches each are issued back to back on a private stream, with a
-    HIP event recorded on that stream at every region boundary; the reported time per launch is the
-    MEDIAN region's event time / K (it includes the gaps between consecutive launches and the cost of
-    the event markers, so it is a lower bound on the in-kernel rate); ms_per_step is the host wall
-    clock over all regions / launches, bracketed by synchronize on both sides;
+  * after W warm-up launches and a synchronize, a gate of plain copies keeps the device busy while the
+    host enqueues everything behind it: a few untimed lead-in launches and then several regions of
+    exactly K launches each, back to back on a private stream, with a HIP event recorded on that stream
+    at every region boundary; the reported time per launch is the MEDIAN region's event time / K (it
+    includes the gaps between consecutive launches and the cost of the event markers, so it is a lower
+    bound on the in-kernel rate); `queued_before_start` says that the host had enqueued every timed launch
+    before the device left the gate, i.e. that the launches really ran back to back (under a profiler the
+    host needs 10+ us per launch and short kernels would otherwise each start on an idle device);
+    ms_per_step is the host wall clock from the first enqueue to the final synchronize, minus the gate's
+    event-measured time, over the timed launches;
   * achieved = algorithmic bytes per launch (each operand once: compulsory reads + writes) / time;
   * roofline.traffic = HBM bytes per launch from rocprofv3 counters, read from
     profiles/hbm_traffic_per_launch.json (written by `python -m inferspore_amd.profile_summary`);
@@ -364,6 +368,11 @@ def make_workloads(torch, lib, stream_handle, rotate):
 
     table = [
         (HEADLINE, lambda: norm(HEADLINE, 2048, 4096, torch.float16, True)),
+        # the same kernel at the row counts a prefill layer hands it (the ragged batch's 2977 valid tokens; 4096)
+        ("fused_add_bias_residual_rmsnorm_f16_2977x4096",
+         lambda: norm("fused_add_bias_residual_rmsnorm_f16_2977x4096", 2977, 4096, torch.float16, True)),
+        ("fused_add_bias_residual_rmsnorm_f16_4096x4096",
+         lambda: norm("fused_add_bias_residual_rmsnorm_f16_4096x4096", 4096, 4096, torch.float16, True)),
         ("rmsnorm_f32_64x4096", lambda: norm("rmsnorm_f32_64x4096", 64, 4096, torch.float32, False)),
         ("rmsnorm_f32_16384x4096", lambda: norm("rmsnorm_f32_16384x4096", 16384, 4096, torch.float32, False)),
         ("embedding_f16_8192x4096_v32000", embedding),
@@ -399,49 +408,147 @@ def region_count(steps, requested):
     return max(5, -(-300 // max(steps, 1)))
 
 
-def time_workload(torch, w, steps, warmup, regions, stream):
-    """W warm-up launches, synchronize, then `regions` back-to-back regions of exactly `steps` launches
-    with an event at every boundary.  Returns (wall ms per launch over all regions, median region's
-    event ms per launch, fastest, slowest)."""
+class QueueGate:
+    """Keeps the device busy with plain copies while the host enqueues a workload's timed launches.
+
+    The timed launches are meant to run back to back.  That only happens while the host enqueues faster
+    than the device executes: a 3-12 us kernel launched from a Python loop is at that edge already, and
+    under a profiler (whose interception costs the host 10+ us per launch) every such kernel starts on
+    an idle device -- its duration then includes the start-up that a busy queue hides behind the previous
+    kernel's tail (12.1-12.3 us instead of 11.3 us for the 2048 x 4096 fp16 fused norm), and the trace
+    and the events disagree.  So each timed pass is preceded by G launches of a large copy (2 GiB of
+    traffic, about a third of a millisecond each: few packets, because the launch queue is finite), G
+    sized so that the copies outlast the host's enqueuing of every timed launch behind them.  A region
+    counts as `queued` when the host had enqueued all of it before the device reached it."""
+    BYTES = 1 << 30
+    MAX_MS = 200.0
+
+    def __init__(self, torch, lib, stream):
+        self.torch, self.lib, self.stream, self.handle = torch, lib, stream, stream.cuda_stream
+        with torch.cuda.stream(stream):
+            self.src = torch.empty(self.BYTES, dtype=torch.uint8, device="cuda").fill_(3)
+            self.dst = torch.empty(self.BYTES, dtype=torch.uint8, device="cuda")
+        self.args = (self.dst.data_ptr(), self.src.data_ptr(), self.BYTES, self.handle)
+        stream.synchronize()
+        n = self.CALIBRATION_LAUNCHES - 2
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        self.launch(2)
+        stream.synchronize()
+        e0.record(stream)
+        t0 = time.perf_counter()
+        self.launch(n)
+        t1 = time.perf_counter()
+        e1.record(stream)
+        stream.synchronize()
+        self.device_us = e0.elapsed_time(e1) * 1e3 / n    # one gate copy on the device
+        self.host_us = (t1 - t0) * 1e6 / n                # one launch's host cost in this process (profiler included)
+
+    CALIBRATION_LAUNCHES = 18
+
+    def launch(self, n):
+        fn, args = self.lib.isp_calibration_copy, self.args
+        for _ in range(n):
+            fn(*args)
+
+    def count(self, timed_launches, host_us):
+        """Gate launches that outlast the host's enqueuing of themselves and of `timed_launches` more."""
+        host_us = max(host_us, self.host_us)
+        need_us = 1.3 * timed_launches * host_us + 200.0
+        return min(int(need_us / self.device_us) + 2, int(self.MAX_MS * 1e3 / self.device_us))
+
+
+PROBE = 16    # untimed launches after the warm-up whose enqueuing is timed on the host (to size the gate)
+
+
+def time_workload(torch, w, steps, warmup, regions, stream, gate):
+    """W warm-up launches, synchronize, the queue gate, then `regions` back-to-back regions of exactly
+    `steps` launches with an event at every boundary.  Returns a dict: wall ms per launch over all regions
+    (gate excluded), the median region's event ms per launch (over the regions in which the host stayed
+    ahead of the device, when there are at least three such), fastest, slowest, and the launches issued in
+    order (for the dispatch log)."""
+    issued = []
+    n_timed = regions * steps + LEAD_IN
     with torch.cuda.stream(stream):
         w.reset()
         for i in range(warmup):
             w.launch(i)
         stream.synchronize()
-        w.reset()
-        torch.cuda.synchronize()
-        ev = [torch.cuda.Event(enable_timing=True) for _ in range(regions + 1)]
-        n = 0
+        # what one launch costs the host in this process, measured on an empty queue once everything
+        # lazy has happened (under a profiler this is 10+ us)
         t0 = time.perf_counter()
-        for _ in range(LEAD_IN):
-            w.launch(n)
-            n += 1
-        for r in range(regions):
-            ev[r].record(stream)
-            for _ in range(steps):
+        for i in range(PROBE):
+            w.launch(i)
+        host_us = (time.perf_counter() - t0) * 1e6 / PROBE
+        stream.synchronize()
+        issued.append(("warmup", warmup + PROBE))
+        for attempt in range(2):
+            w.reset()
+            torch.cuda.synchronize()
+            g = gate.count(n_timed, host_us)
+            ev = [torch.cuda.Event(enable_timing=True) for _ in range(regions + 1)]
+            eg = torch.cuda.Event(enable_timing=True)
+            host_at = [0.0] * (regions + 1)
+            n = 0
+            t0 = time.perf_counter()
+            eg.record(stream)
+            gate.launch(g)
+            for _ in range(LEAD_IN):
                 w.launch(n)
                 n += 1
-        ev[regions].record(stream)
-        stream.synchronize()
-        torch.cuda.synchronize()
-        t1 = time.perf_counter()
-    per = sorted(ev[r].elapsed_time(ev[r + 1]) / steps for r in range(regions))
-    wall_ms = (t1 - t0) * 1e3 / (regions * steps + LEAD_IN)
-    return wall_ms, per[len(per) // 2], per[0], per[-1]
+            for r in range(regions):
+                host_at[r] = time.perf_counter()
+                ev[r].record(stream)
+                for _ in range(steps):
+                    w.launch(n)
+                    n += 1
+            host_at[regions] = time.perf_counter()
+            ev[regions].record(stream)
+            stream.synchronize()
+            torch.cuda.synchronize()
+            t1 = time.perf_counter()
+            dev_at = [eg.elapsed_time(e) for e in ev]    # ms after the gate began on the device
+            gate_ms = dev_at[0]                          # gate copies + lead-in launches
+            per_all = [(dev_at[r + 1] - dev_at[r]) / steps for r in range(regions)]
+            # The device cannot reach `eg` before t0, so it began region r no earlier than t0 + dev_at[r].
+            # The host stayed ahead throughout region r if it began enqueuing the region before the device
+            # began it and enqueued its last launch before the device began that one (rates in between are
+            # steady, and a host that blocks does so on a full queue).
+            ahead = [(host_at[r] - t0) * 1e3 < dev_at[r] and
+                     (host_at[r + 1] - t0) * 1e3 < dev_at[r + 1] - per_all[r] for r in range(regions)]
+            enqueue_us = (host_at[regions] - t0) * 1e6 / (g + n)
+            issued.append(("gate", g))
+            if sum(ahead) >= min(3, regions) or attempt == 1:
+                issued.append(("timed", n))
+                break
+            issued.append(("discarded", n))
+            host_us = 2.0 * max(host_us, (host_at[regions] - host_at[0]) * 1e6 / (regions * steps))
+    good = [t for t, q in zip(per_all, ahead) if q]
+    per = sorted(good if len(good) >= min(3, regions) else per_all)
+    # the device is busy from the first gate copy to the last timed launch: what the wall clock saw beyond
+    # the gate (and the lead-in, a few launches) is the timed launches plus the submit and wake-up latencies
+    wall_ms = max((t1 - t0) * 1e3 - gate_ms, 0.0) / (regions * steps)
+    return {"wall_ms": wall_ms, "event_ms": per[len(per) // 2], "fastest": per[0], "slowest": per[-1],
+            "queued_before_start": (host_at[regions] - t0) * 1e3 < gate_ms, "regions_ahead": ahead,
+            "gate_launches": g, "issued": issued, "host_enqueue_us_per_launch": enqueue_us,
+            "host_us_per_launch_empty_queue": host_us}
 
 
-def measure(torch, w, steps, warmup, regions, stream, traffic):
-    wall_ms, event_ms, fastest, slowest = time_workload(torch, w, steps, warmup, regions, stream)
+def measure(torch, w, steps, warmup, regions, stream, traffic, gate):
+    t = time_workload(torch, w, steps, warmup, regions, stream, gate)
+    event_ms = t["event_ms"]
     gbs = w.bytes_per_launch / (event_ms * 1e-3) / 1e9
     return {
         "workload": w.name, "kernel": w.kernel, "dtype": w.dtype, "tokens": w.tokens, "buffer_sets": w.sets,
         "algorithmic_bytes": w.bytes_per_launch, "launches_per_step": w.launches_per_step,
-        "ms_per_step_wall": wall_ms, "ms_per_launch_events": event_ms,
-        "ms_fastest_region": fastest, "ms_slowest_region": slowest, "regions": regions,
+        "ms_per_step_wall": t["wall_ms"], "ms_per_launch_events": event_ms,
+        "ms_fastest_region": t["fastest"], "ms_slowest_region": t["slowest"], "regions": regions,
         "GBps": gbs, "frac_of_hbm_peak": gbs / HBM_PEAK_GBS,
         "tokens_per_s": (w.tokens / (event_ms * 1e-3)) if w.tokens else None,
         "traffic": traffic.get(w.name),
-        "launches_total": warmup + LEAD_IN + regions * steps,
+        "queued_before_start": t["queued_before_start"], "regions_queued": sum(t["regions_ahead"]),
+        "regions_ahead": t["regions_ahead"], "gate_launches": t["gate_launches"],
+        "host_enqueue_us_per_launch": t["host_enqueue_us_per_launch"],
+        "issued": t["issued"],
     }
 
 
@@ -745,6 +852,8 @@ def compact(r):
         out["tokens_per_s"] = round(r["tokens_per_s"])
     if r["launches_per_step"] != 1:
         out["launches_per_step"] = r["launches_per_step"]
+    if r.get("regions_queued", r["regions"]) < r["regions"]:
+        out["regions_queued"] = r["regions_queued"]   # of r["regions"]: the host fell behind the device in the others
     return out
 
 
@@ -768,6 +877,16 @@ def main():
     traffic = measured_traffic()
     dispatch_log = []
 
+    def log_issued(name, w, issued):
+        """Every launch of a workload's measurement in order: warm-up, gate copies, timed launches (the first
+        LEAD_IN of them untimed); a pass that was repeated with a longer gate is logged as discarded."""
+        for kind, count in issued:
+            if kind == "gate":
+                dispatch_log.append(["gate", "isp::copy_vec<1>", count])
+            else:
+                dispatch_log.append([name if kind == "timed" else kind + ":" + name, w.kernel,
+                                     count * w.launches_per_step])
+
     def run_all(rotate, names=None):
         out = []
         for name, make in make_workloads(torch, lib, handle, rotate):
@@ -778,9 +897,9 @@ def main():
             with torch.cuda.stream(stream):
                 w = make()
             torch.cuda.synchronize()
-            r = measure(torch, w, a.steps, a.warmup, regions, stream, traffic)
+            r = measure(torch, w, a.steps, a.warmup, regions, stream, traffic, gate)
             out.append(r)
-            dispatch_log.append([name, w.kernel, r["launches_total"] * w.launches_per_step])
+            log_issued(name, w, r.pop("issued"))
             # the buffers go back to torch's caching allocator, not to the driver: kernels that run
             # on freshly mapped device memory measured up to 2x slower at launch-bound sizes
             del w
@@ -796,6 +915,8 @@ def main():
         stream.synchronize()
         del a_buf, b_buf
     dispatch_log.append(["device_warmup", "isp::copy_vec<1>", 2000])
+    gate = QueueGate(torch, lib, stream)
+    dispatch_log.append(["gate_calibration", "isp::copy_vec<1>", QueueGate.CALIBRATION_LAUNCHES])
 
     if a.copy_curve:
         points = []
@@ -803,7 +924,7 @@ def main():
             with torch.cuda.stream(stream):
                 w = make_copy_workload(torch, lib, handle, (mib << 20) // 2)
             torch.cuda.synchronize()
-            r = measure(torch, w, a.steps, a.warmup, regions, stream, traffic)
+            r = measure(torch, w, a.steps, a.warmup, regions, stream, traffic, gate)
             points.append({"traffic_MiB": mib, "us_per_launch": r["ms_per_launch_events"] * 1e3, "GBps": r["GBps"],
                            "frac_of_hbm_peak": r["frac_of_hbm_peak"]})
             del w
@@ -846,6 +967,8 @@ def main():
         line["kernels"] = results
     if a.kernels_only:
         line["dispatch_log"] = dispatch_log
+        line["lead_in"] = LEAD_IN
+        line["regions_ahead"] = {r["workload"]: r["regions_ahead"] for r in results}
     if not a.only and not a.kernels_only:
         layer = context_layer_record(torch, a.steps, a.warmup, stream)
         own = {"qkv_bias_rope_transpose_f16_b8_s512": 1, "concat_kv_cache_f16_b8_q512_S1024": 1,
@@ -882,6 +1005,9 @@ def main():
                      "avg_launch_ms": head["ms_per_launch_events"],
                      "fastest_region_ms": head["ms_fastest_region"], "slowest_region_ms": head["ms_slowest_region"],
                      "vs_copy": head.get("vs_copy"),
+                     "queued_before_start": head["queued_before_start"], "regions_queued": head["regions_queued"],
+                     "regions": head["regions"], "gate_launches": head["gate_launches"],
+                     "host_enqueue_us_per_launch": round(head["host_enqueue_us_per_launch"], 2),
                      "per_config": {r["workload"]: compact(r) for r in results}},
     })
     if not a.no_cpu and not a.kernels_only:

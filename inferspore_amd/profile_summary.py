@@ -102,31 +102,62 @@ def main():
     per_config = bench["roofline"]["per_config"]
     log = bench["dispatch_log"]
     rows = library_rows(find_one(tdir, "*kernel_trace.csv"))
-    dur = attribute(rows, log, lambda r: int(r["End_Timestamp"]) - int(r["Start_Timestamp"]))
-    warm = bench["warmup"]
+    # gap between a dispatch's start and the end of the dispatch before it (this library's kernels only;
+    # nothing else runs inside a timed pass)
+    prev_end = None
+    for r in rows:
+        r["_gap"] = (int(r["Start_Timestamp"]) - prev_end) if prev_end is not None else 0
+        prev_end = int(r["End_Timestamp"])
+    dur = attribute(rows, log, lambda r: (int(r["End_Timestamp"]) - int(r["Start_Timestamp"]), r["_gap"]))
+    # the dispatch log lists warm-up, gate and timed launches separately; the first `lead_in` timed launches are untimed
+    warm = bench.get("lead_in", bench["warmup"])
+    steps = bench["steps"]
+    ahead_of = bench.get("regions_ahead", {})
+
+    def in_ahead_regions(v, workload, per_step):
+        """The dispatches of the regions in which the host stayed ahead of the device (the ones the benchmark's
+        median is taken over); all timed dispatches if the benchmark did not say."""
+        flags = ahead_of.get(workload)
+        if not flags or sum(flags) < min(3, len(flags)):
+            return tail_of(v, warm * per_step)
+        sel = []
+        for r, ok in enumerate(flags):
+            if ok:
+                sel += v[(warm + r * steps) * per_step:(warm + (r + 1) * steps) * per_step]
+        return sel
+
     out = ["rocprofv3 kernel-trace summary: every kernel of the library at its benchmark shape (bench.py, all workloads)", "",
            "command (run from /tmp with TMPDIR=/tmp on the MI355X box):",
            "  rocprofv3 --kernel-trace --stats --output-format csv -d RUN/trace -o bench -- python3 bench.py --kernels-only",
            "  python3 -m inferspore_amd.profile_summary RUN --out profiles",
-           "  (--steps %d --warmup %d; launches rotate over >1 GiB of buffer sets; warm-up dispatches excluded below)"
-           % (bench["steps"], warm), "",
-           "per workload from the kernel trace -- durations in microseconds; GB/s = algorithmic bytes / average duration;",
-           "`events` = the benchmark's own HIP-event time per launch in the same (profiled) run",
-           "%-48s %-50s %6s %8s %8s %8s %8s %7s %8s" % ("workload", "kernel", "calls", "avg_us", "med_us", "min_us",
-                                                         "max_us", "GB/s", "events")]
+           "  (--steps %d --warmup %d; launches rotate over >1 GiB of buffer sets; warm-up, gate and lead-in dispatches excluded)"
+           % (steps, bench["warmup"]), "",
+           "per workload from the kernel trace -- durations in microseconds; GB/s = algorithmic bytes / average duration.",
+           "calls .. max_us cover the dispatches of the timed regions in which the host stayed ahead of the device, i.e. the",
+           "launches that ran back to back -- the same regions the benchmark's median is taken over (`regions` = how many of",
+           "the timed regions those are; under the profiler a launch costs the host 12 us, so it falls behind on short kernels).",
+           "`events` = the benchmark's own HIP-event time per launch in the same (profiled) run; `idle_us` (`n`) = average",
+           "duration of the timed dispatches that started 1 us or more after the previous one had ended, i.e. on an idle device.",
+           "%-48s %-50s %7s %6s %8s %8s %8s %8s %7s %8s %8s %5s" % (
+               "workload", "kernel", "regions", "calls", "avg_us", "med_us", "min_us", "max_us", "GB/s", "events", "idle_us", "n")]
     for workload, kernel, _ in log:
         if workload not in per_config:
             continue
         rec = per_config[workload]
         parts = dur[workload]
         steps_per = rec.get("launches_per_step", 1)
-        for b, v in parts.items():
-            v = tail_of(v, warm)
+        flags = ahead_of.get(workload)
+        reg = ("%d/%d" % (sum(flags), len(flags))) if flags else "-"
+        for b, pairs in parts.items():
+            v = [d for d, _ in in_ahead_regions(pairs, workload, 1)]
+            idle = [d for d, g in tail_of(pairs, warm) if g >= 1000]
             avg = sum(v) / len(v)
             full = [k for k in kernel.split(" + ") if base_name(k) == b][0]
             gbs = ("%7.0f" % (rec["bytes"] / avg)) if steps_per == 1 else "      -"
-            out.append("%-48s %-50s %6d %8.2f %8.2f %8.2f %8.2f %s %8.2f" % (
-                workload, full[:50], len(v), avg / 1e3, median(v) / 1e3, min(v) / 1e3, max(v) / 1e3, gbs, rec["us"]))
+            idle_s = ("%8.2f %5d" % (sum(idle) / len(idle) / 1e3, len(idle))) if idle else "       - %5d" % 0
+            out.append("%-48s %-50s %7s %6d %8.2f %8.2f %8.2f %8.2f %s %8.2f %s" % (
+                workload, full[:50], reg, len(v), avg / 1e3, median(v) / 1e3, min(v) / 1e3, max(v) / 1e3, gbs,
+                rec["us"], idle_s))
     stats = find_one(tdir, "*kernel_stats.csv")
     out += ["", "rows of the --stats table for this library's kernels (Name, Calls, AverageNs, MinNs, MaxNs; kernels used by",
             "several workloads and the device warm-up copies are merged in these rows):"]
@@ -146,7 +177,8 @@ def main():
         b = load_bench(d)
         rows = library_rows(find_one(d, "*counter_collection.csv"), name)
         vals = attribute(rows, b["dispatch_log"], lambda r: float(r["Counter_Value"]))
-        return {w: sum(median(tail_of(v, b["warmup"])) for v in parts.values()) for w, parts in vals.items()}, b
+        return {w: sum(median(tail_of(v, b.get("lead_in", b["warmup"]))) for v in parts.values())
+                for w, parts in vals.items() if parts}, b
 
     fetch, write = counter_medians("FETCH_SIZE"), counter_medians("WRITE_SIZE")
     if fetch and write:
