@@ -119,12 +119,15 @@ class Workload:
 
 
 def norm_kernel_name(lib, es, tokens, hidden, fused):
+    """The instantiation the launcher picks (`fused`: with residual and bias, as the benchmark's fused rows are)."""
     v = [ctypes.c_int() for _ in range(4)]
     rc = lib.isp_norm_launch_config(es, tokens, hidden, int(fused), *[ctypes.byref(x) for x in v])
     if rc:
         return "isp::fused_norm_generic"
-    return "isp::fused_norm_rows<%s, %d, %d, %d, %d>" % ("__half" if es == 2 else "float", v[1].value, v[0].value,
-                                                          v[3].value, v[2].value)
+    t = "__half" if es == 2 else "float"
+    if lib.isp_norm_launch_variant(es, tokens, hidden, int(fused), int(fused), 0) == 1:
+        return "isp::fused_norm_few_rows<%s, %d, %d, %d, %d>" % (t, v[1].value, v[0].value, v[3].value, 2 if fused else 0)
+    return "isp::fused_norm_rows<%s, %d, %d, %d, %d>" % (t, v[1].value, v[0].value, v[3].value, v[2].value)
 
 
 def make_copy_workload(torch, lib, stream_handle, nbytes, rotate=True):

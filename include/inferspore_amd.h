@@ -276,10 +276,18 @@ int isp_calibration_copy(void* dst, const void* src, size_t bytes, isp_stream_t 
 int isp_norm_launch_config(int elem_size, int tokens, int hidden, int fused, int* waves_per_row,
                            int* vectors_per_lane, int* block_threads, int* store_kind);
 
+/* isp_norm_launch_variant: 1 if a call with these operands (`flags` as for the fused entry point) is launched
+ *   as isp::fused_norm_few_rows -- the same row algorithm with the operand set fixed at compile time, taken by
+ *   launches that occupy less than a quarter of the device (every decode-step norm) -- and 0 if as the general
+ *   isp::fused_norm_rows; the waves per row, vectors per lane and store kind are those of
+ *   isp_norm_launch_config, the workgroup is max(256, 64 x waves per row) threads.  No counterpart in the
+ *   reference (its launcher has one configuration, src/kernels/fused_addresidual_norm.cu:155-159). */
+int isp_norm_launch_variant(int elem_size, int tokens, int hidden, int has_residual, int has_bias, unsigned flags);
+
 typedef enum isp_tuning_knob {
     ISP_TUNE_NORM_WAVES_PER_ROW = 0, /* 1, 2, 4, 8 or 16 waves cooperate on one token row */
-    ISP_TUNE_NORM_STORE = 1,         /* output stores: 1 = plain, 2 = non-temporal (default),
-                                        3 = non-temporal write-through */
+    ISP_TUNE_NORM_STORE = 1,         /* output stores: 1 = plain (default where a launch writes at most 1 MiB),
+                                        2 = non-temporal (default otherwise), 3 = non-temporal write-through */
     ISP_TUNE_SWIGLU_UNROLL = 2,      /* 1 (default), 2 or 4 vector pairs in flight per lane */
     ISP_TUNE_SWIGLU_STORE = 3,       /* 1 = plain, 2 = non-temporal (default), 3 = write-through */
     ISP_TUNE_EMBED_VARIANT = 4,      /* 1 = a wave per row, 2 = a workgroup per row,
@@ -295,7 +303,8 @@ typedef enum isp_tuning_knob {
     ISP_TUNE_NORM_BLOCK_THREADS = 8, /* 256, 512 or 1024 threads per workgroup (several token rows share a
                                         workgroup when a row needs fewer); 0 = automatic */
     ISP_TUNE_NORM_ORDER = 9,         /* 2 = streaming (each vector processed, and the residual stored, as it
-                                        arrives); 0, 1 = read everything, then write everything (default) */
+                                        arrives); 0, 1 = read everything, then write everything (default);
+                                        3 = as 0, but launches of a few rows also take the general kernel */
     ISP_TUNE_MOVER_BLOCK_THREADS = 10, /* KV append / broadcast: 256, 512 or 1024 threads per workgroup */
     ISP_TUNE_COUNT = 11
 } isp_tuning_knob;

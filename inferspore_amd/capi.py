@@ -50,6 +50,7 @@ SIGNATURES = {
     "isp_tuning_set": (_i, [_i, _i]),
     "isp_calibration_copy": (_i, [_vp, _vp, C.c_size_t, _vp]),
     "isp_norm_launch_config": (_i, [_i, _i, _i, _i] + [C.POINTER(C.c_int)] * 4),
+    "isp_norm_launch_variant": (_i, [_i, _i, _i, _i, _i, C.c_uint]),
 }
 
 _lib = None

@@ -49,10 +49,13 @@ __device__ __forceinline__ float tree_sum(const float* p) {
 // plain RMSNorm, and 8-12 % slower for 32-bit rows with a residual.  Same bits under both.
 constexpr unsigned kNormStreamingOrder = 0x80000000u;
 
-template <typename T, int NV, int WPR, int ST, int BLOCK>
-__global__ __launch_bounds__(BLOCK) void fused_norm_rows(T* residual, T* out, const T* bias,
-                                                         const T* gamma, float eps, int tokens,
-                                                         int hidden, unsigned flags) {
+// Which operands exist: known only at run time (the general kernel: uniform scalar branches), or fixed at
+// compile time for the kernels that launches of a few rows take (fused_norm_few_rows).
+constexpr int kOpsRuntime = -1, kOpsNone = 0, kOpsResidual = 1, kOpsResidualBias = 2;
+
+template <typename T, int NV, int WPR, int ST, int BLOCK, int OPS>
+__device__ __forceinline__ void norm_rows_body(T* residual, T* out, const T* bias, const T* gamma, float eps,
+                                               int tokens, int hidden, unsigned flags) {
     constexpr int VEC = Elem<T>::kVec;
     constexpr int ROW_THREADS = kWave * WPR;
     static_assert(BLOCK >= norm_block(WPR) && BLOCK % ROW_THREADS == 0, "workgroup must hold whole rows");
@@ -63,9 +66,10 @@ __global__ __launch_bounds__(BLOCK) void fused_norm_rows(T* residual, T* out, co
     const int row = blockIdx.x * ROWS + slot;
     const bool live = row < tokens;  // uniform within a wave
     const int nvec = hidden / VEC;
-    const bool has_res = residual != nullptr, has_bias = bias != nullptr;  // uniform: scalar branches
-    const bool literal_order = (flags & ISP_NORM_RESIDUAL_EXCLUDES_BIAS) != 0;
-    const bool streaming = (flags & kNormStreamingOrder) != 0;
+    const bool has_res = OPS == kOpsRuntime ? residual != nullptr : OPS >= kOpsResidual;  // uniform: scalar branches
+    const bool has_bias = OPS == kOpsRuntime ? bias != nullptr : OPS == kOpsResidualBias;
+    const bool literal_order = OPS == kOpsRuntime && (flags & ISP_NORM_RESIDUAL_EXCLUDES_BIAS) != 0;
+    const bool streaming = OPS == kOpsRuntime && (flags & kNormStreamingOrder) != 0;
     const size_t base = (size_t)(live ? row : 0) * (size_t)hidden;
     T* out_row = out + base;
     T* rsd_row = residual + base;  // dereferenced only when has_res
@@ -175,6 +179,29 @@ __global__ __launch_bounds__(BLOCK) void fused_norm_rows(T* residual, T* out, co
             store16_sel<ST>(out_row + (size_t)(lane + j * ROW_THREADS) * VEC, Elem<T>::pack(y));
         }
     }
+}
+
+template <typename T, int NV, int WPR, int ST, int BLOCK>
+__global__ __launch_bounds__(BLOCK) void fused_norm_rows(T* residual, T* out, const T* bias,
+                                                         const T* gamma, float eps, int tokens,
+                                                         int hidden, unsigned flags) {
+    norm_rows_body<T, NV, WPR, ST, BLOCK, kOpsRuntime>(residual, out, bias, gamma, eps, tokens, hidden, flags);
+}
+
+// The same row algorithm for launches of a few rows (every decode-step norm).  Such a launch is a chain of
+// latencies, not a stream: the device is mostly empty, nothing hides an instruction, and what the general
+// kernel pays for deciding at run time which operands exist and in which order to store (branches, selects,
+// and waits that must assume the worst because loads sit inside branches) is on the critical path -- 64 x
+// 4096 fp32: 2.9 us per launch back to back with the general kernel, 2.5 us with the operands fixed at
+// compile time, against 2.4 us for a copy of the same bytes.  One row per workgroup of WPR waves, one or two
+// vectors per lane, the default residual order only.  Same operations in the same order, so the same bits.
+// (Requesting gamma and bias together with the row, to take a cache round trip out of the chain, measured
+// 0.05-0.2 us SLOWER at 16-256 rows, twice, in this kernel and in a stripped-down one.)
+template <typename T, int NV, int WPR, int ST, int OPS>
+__global__ __launch_bounds__(norm_block(WPR)) void fused_norm_few_rows(T* residual, T* out, const T* bias,
+                                                                       const T* gamma, float eps, int tokens,
+                                                                       int hidden) {
+    norm_rows_body<T, NV, WPR, ST, norm_block(WPR), OPS>(residual, out, bias, gamma, eps, tokens, hidden, 0u);
 }
 
 // Any hidden size and any alignment: one workgroup per row, scalar accesses, two passes over the
@@ -289,14 +316,55 @@ static long long resident_rows(const NormVariant<T>& v) {
 struct NormPlan {
     int wpr, nv, store, block_big;
     bool streaming;  // kNormStreamingOrder
+    bool few;        // the launch occupies less than a quarter of the device: fused_norm_few_rows if it has the shape
 };
+
+template <typename T>
+using NormFewKernel = void (*)(T*, T*, const T*, const T*, float, int, int);
+
+template <typename T, int NV, int WPR, int ST>
+static NormFewKernel<T> few_ops(int ops) {
+    if (ops == kOpsNone) return fused_norm_few_rows<T, NV, WPR, ST, kOpsNone>;
+    if (ops == kOpsResidual) return fused_norm_few_rows<T, NV, WPR, ST, kOpsResidual>;
+    return fused_norm_few_rows<T, NV, WPR, ST, kOpsResidualBias>;
+}
+
+// The few-rows instantiation for (waves per row, vectors per lane, store kind, operands), or nullptr: one
+// vector per lane with any number of waves per row, two only with 16 waves (rows are split as far as they
+// go before a lane takes a second vector); plain or non-temporal stores.
+template <typename T>
+static NormFewKernel<T> norm_few_variant(int wpr, int nv, int st, int ops) {
+    if (st != kStorePlain && st != kStoreStream) return nullptr;
+    const bool plain = st == kStorePlain;
+    if (nv == 2 && wpr == 16)
+        return plain ? few_ops<T, 2, 16, kStorePlain>(ops) : few_ops<T, 2, 16, kStoreStream>(ops);
+    if (nv != 1) return nullptr;
+    switch (wpr) {
+        case 1: return plain ? few_ops<T, 1, 1, kStorePlain>(ops) : few_ops<T, 1, 1, kStoreStream>(ops);
+        case 2: return plain ? few_ops<T, 1, 2, kStorePlain>(ops) : few_ops<T, 1, 2, kStoreStream>(ops);
+        case 4: return plain ? few_ops<T, 1, 4, kStorePlain>(ops) : few_ops<T, 1, 4, kStoreStream>(ops);
+        case 8: return plain ? few_ops<T, 1, 8, kStorePlain>(ops) : few_ops<T, 1, 8, kStoreStream>(ops);
+        case 16: return plain ? few_ops<T, 1, 16, kStorePlain>(ops) : few_ops<T, 1, 16, kStoreStream>(ops);
+        default: return nullptr;
+    }
+}
+
+// Operand combination of a call as the few-rows kernels know them, or kOpsRuntime if they do not.
+inline int few_rows_ops(bool has_res, bool has_bias, unsigned flags) {
+    if (flags & ISP_NORM_RESIDUAL_EXCLUDES_BIAS) return kOpsRuntime;
+    if (!has_res) return has_bias ? kOpsRuntime : kOpsNone;
+    return has_bias ? kOpsResidualBias : kOpsResidual;
+}
 
 // The launch configuration for `tokens` rows of `nvec` 16-byte vectors.
 template <typename T>
 static NormPlan plan_norm(int tokens, int nvec, bool fused) {
     auto vectors_per_lane = [nvec](int w) { return (nvec + kWave * w - 1) / (kWave * w); };
-    // in place on both tensors: plain non-temporal stores measured best (write-through costs 2 %)
-    const int kind = store_kind(tuning(ISP_TUNE_NORM_STORE), kStoreStream);
+    // in place on both tensors: plain non-temporal stores measured best (write-through costs 2 %) -- except
+    // where a launch writes no more than 1 MiB: ordinary stores, which the L2 acknowledges, then end the
+    // kernel sooner (16 x 4096 fp32: 2.13 against 2.56 us per launch; equal at 1 MiB; 2 % slower at 2 MiB)
+    const size_t written = (size_t)tokens * (size_t)nvec * 16u * (fused ? 2u : 1u);
+    const int kind = store_kind(tuning(ISP_TUNE_NORM_STORE), written <= (1u << 20) ? kStorePlain : kStoreStream);
     const int block_knob = tuning(ISP_TUNE_NORM_BLOCK_THREADS);
     int wpr = tuning(ISP_TUNE_NORM_WAVES_PER_ROW);
     if (wpr != 1 && wpr != 2 && wpr != 4 && wpr != 8 && wpr != 16) {
@@ -343,8 +411,10 @@ static NormPlan plan_norm(int tokens, int nvec, bool fused) {
     // 2048 x 4096 with a residual, 0.5-3 % elsewhere; with 32-bit elements, and with one wave per
     // row, the 256-thread workgroup measured 1-6 % faster)
     const bool big = block_knob >= 512 || (block_knob <= 0 && (wpr == 4 || wpr == 2) && sizeof(T) == 2);
-    const bool streaming = tuning(ISP_TUNE_NORM_ORDER) == 2;
-    return {wpr, vectors_per_lane(wpr), kind, big ? 1 : 0, streaming};
+    const int order = tuning(ISP_TUNE_NORM_ORDER);
+    const bool streaming = order == 2;
+    const bool few = !streaming && order != 3 && (long long)tokens * wpr * 4 <= (long long)resident_waves();
+    return {wpr, vectors_per_lane(wpr), kind, big ? 1 : 0, streaming, few};
 }
 
 template <typename T>
@@ -368,11 +438,19 @@ static int fused_norm(void* residual_, void* out_, const void* bias_, const void
                            residual, out, bias, gamma, eps, tokens, hidden, flags & ~kNormStreamingOrder);
     } else {
         const NormPlan plan = plan_norm<T>(tokens, hidden / VEC, residual != nullptr);
-        const NormVariant<T> v = norm_variant<T>(plan.wpr, plan.nv, plan.store, plan.block_big != 0);
-        const dim3 grid((unsigned)((tokens + v.rows_per_block - 1) / v.rows_per_block));
-        hipLaunchKernelGGL(v.kernel, grid, dim3(v.block), 0, s, residual, out, bias, gamma, eps,
-                           tokens, hidden,
-                           (flags & ~kNormStreamingOrder) | (plan.streaming ? kNormStreamingOrder : 0u));
+        const int ops = few_rows_ops(residual != nullptr, bias != nullptr, flags);
+        const NormFewKernel<T> few =
+            plan.few && ops != kOpsRuntime ? norm_few_variant<T>(plan.wpr, plan.nv, plan.store, ops) : nullptr;
+        if (few != nullptr) {
+            const int block = norm_block(plan.wpr), rows_per_block = block / (kWave * plan.wpr);
+            hipLaunchKernelGGL(few, dim3((unsigned)((tokens + rows_per_block - 1) / rows_per_block)), dim3(block), 0,
+                               s, residual, out, bias, gamma, eps, tokens, hidden);
+        } else {
+            const NormVariant<T> v = norm_variant<T>(plan.wpr, plan.nv, plan.store, plan.block_big != 0);
+            const dim3 grid((unsigned)((tokens + v.rows_per_block - 1) / v.rows_per_block));
+            hipLaunchKernelGGL(v.kernel, grid, dim3(v.block), 0, s, residual, out, bias, gamma, eps, tokens, hidden,
+                               (flags & ~kNormStreamingOrder) | (plan.streaming ? kNormStreamingOrder : 0u));
+        }
     }
     return note_launch(hipGetLastError());
 }
@@ -391,9 +469,26 @@ static int describe_plan(int tokens, int hidden, int fused, int* wpr, int* nv, i
     return ISP_OK;
 }
 
+// 1 if a call with these operands takes a few-rows kernel, 0 if the general one, < 0 if neither applies.
+template <typename T>
+static int describe_variant(int tokens, int hidden, int has_residual, int has_bias, unsigned flags) {
+    constexpr int VEC = Elem<T>::kVec;
+    if (tokens <= 0 || hidden <= 0) return ISP_ERR_BAD_SHAPE;
+    if (hidden % VEC != 0 || hidden / VEC > kMaxNv * kWave * kMaxWpr) return ISP_ERR_UNSUPPORTED;
+    const NormPlan plan = plan_norm<T>(tokens, hidden / VEC, has_residual != 0);
+    const int ops = few_rows_ops(has_residual != 0, has_bias != 0, flags);
+    return plan.few && ops != kOpsRuntime && norm_few_variant<T>(plan.wpr, plan.nv, plan.store, ops) != nullptr ? 1 : 0;
+}
+
 }  // namespace isp
 
 extern "C" {
+
+int isp_norm_launch_variant(int elem_size, int tokens, int hidden, int has_residual, int has_bias, unsigned flags) {
+    if (elem_size == 2) return isp::describe_variant<__half>(tokens, hidden, has_residual, has_bias, flags);
+    if (elem_size == 4) return isp::describe_variant<float>(tokens, hidden, has_residual, has_bias, flags);
+    return ISP_ERR_BAD_SHAPE;
+}
 
 int isp_norm_launch_config(int elem_size, int tokens, int hidden, int fused, int* waves_per_row,
                            int* vectors_per_lane, int* block_threads, int* store_kind) {

@@ -60,12 +60,71 @@ def test_norm_every_vectors_per_lane_waves_per_row_store_kind_and_workgroup_size
         else:
             assert_f16_close(base[1], e_out, "norm hidden %d" % hidden, max_mismatch_fraction=0.05)
         # the row sum is one fixed tree whatever the split of the row over waves and vectors per lane
-        for split, store, block, order in itertools.product((1, 2, 4, 8, 16), (1, 2, 3), (256, 512), (1, 2)):
+        # order 1: the default (seven rows take the few-rows kernels where one exists), 2: streaming, 3: the general
+        # kernel also for few rows
+        for split, store, block, order in itertools.product((1, 2, 4, 8, 16), (1, 2, 3), (256, 512), (1, 2, 3)):
             say("norm %s hidden=%d waves/row=%d store=%d block=%d order=%d" % (dtype.__name__, hidden, split, store,
                                                                                  block, order))
             got = with_knobs({capi.TUNE_NORM_WAVES_PER_ROW: split, capi.TUNE_NORM_STORE: store,
                               capi.TUNE_NORM_BLOCK_THREADS: block, capi.TUNE_NORM_ORDER: order}, run)
             assert np.array_equal(got[0], base[0]) and np.array_equal(got[1], base[1])
+
+
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+def test_norm_few_rows_kernels_match_the_general_kernel_and_the_oracle(isp, oracle, dtype):
+    """Launches of a few rows take kernels with the operand set fixed at compile time (one or two vectors per
+    lane x waves per row x plain / non-temporal stores x {RMSNorm, residual, residual + bias}); every one of
+    them must give the bits of the general kernel (knob order 3) and match the oracle."""
+    from inferspore_amd import capi
+    lib = capi.lib()
+    vec = 8 if dtype == np.float16 else 4
+    es = 2 if dtype == np.float16 else 4
+    shapes = [(wpr, 1) for wpr in (1, 2, 4, 8, 16)] + [(16, 2)]
+    seen = 0
+    for (wpr, nv), tokens in itertools.product(shapes, (1, 5)):
+        hidden = vec * 64 * wpr * nv - (vec * 3 if wpr * nv > 1 else 0)   # ragged last wave
+        for with_res, with_bias in ((False, False), (True, False), (True, True)):
+            res, out, bias, gamma = norm_inputs(tokens, hidden, dtype, seed=100 * wpr + 10 * nv + tokens)
+            d_bias, d_gamma = (dev(bias) if with_bias else None), dev(gamma)
+
+            def run():
+                d_res, d_out = (dev(res) if with_res else None), dev(out)
+                if with_res:
+                    isp.fused_add_bias_residual_rmsnorm(d_res, d_out, d_bias, d_gamma, 1e-5)
+                else:
+                    isp.rmsnorm(d_out, d_gamma, 1e-5)
+                return (d_res.cpu().numpy() if with_res else None), d_out.cpu().numpy()
+
+            e_res, e_out = oracle.fused_norm(res if with_res else None, out, bias if with_bias else None, gamma, 1e-5)
+            general = with_knobs({capi.TUNE_NORM_WAVES_PER_ROW: wpr, capi.TUNE_NORM_ORDER: 3}, run)
+            if with_res:
+                assert np.array_equal(general[0], e_res)
+            if dtype == np.float32:
+                assert_f32_close(general[1], e_out, "norm hidden %d" % hidden)
+            else:
+                assert_f16_close(general[1], e_out, "norm hidden %d" % hidden, max_mismatch_fraction=0.05)
+            for store in (1, 2):
+                say("few-rows norm %s hidden=%d tokens=%d waves/row=%d residual=%s bias=%s store=%d" % (
+                    dtype.__name__, hidden, tokens, wpr, with_res, with_bias, store))
+                knobs = {capi.TUNE_NORM_WAVES_PER_ROW: wpr, capi.TUNE_NORM_STORE: store}
+
+                def variant():
+                    return lib.isp_norm_launch_variant(es, tokens, hidden, int(with_res), int(with_bias), 0)
+
+                assert with_knobs(knobs, variant) == 1, "this shape must take a few-rows kernel"
+                seen += 1
+                got = with_knobs(knobs, run)
+                if with_res:
+                    assert np.array_equal(got[0], general[0])
+                assert np.array_equal(got[1], general[1])
+    assert seen == len(shapes) * 2 * 3 * 2
+    # what the few-rows kernels do not cover goes to the general kernel: the reference's literal residual order,
+    # a bias without a residual, more than two vectors per lane, write-through stores, many rows
+    assert lib.isp_norm_launch_variant(es, 4, 4096, 1, 1, 1) == 0
+    assert lib.isp_norm_launch_variant(es, 4, 4096, 0, 1, 0) == 0
+    assert lib.isp_norm_launch_variant(es, 4, vec * 64 * 16 * 4, 1, 0, 0) == 0
+    assert lib.isp_norm_launch_variant(es, 16384, 4096, 1, 0, 0) == 0
+    assert with_knobs({capi.TUNE_NORM_STORE: 3}, lambda: lib.isp_norm_launch_variant(es, 4, 4096, 1, 0, 0)) == 0
 
 
 @pytest.mark.parametrize("dtype", [np.float16, np.float32])
