@@ -83,7 +83,10 @@ public:
     LlamaContextDecoderLayer(const LlamaContextDecoderLayer&) = delete;
     LlamaContextDecoderLayer& operator=(const LlamaContextDecoderLayer&) = delete;
 
-    // (Re)allocates the intermediate buffers for these extents; forward() calls it when they grow.
+    // Makes sure every intermediate buffer holds these extents.  Capacities only grow: a buffer is taken from the
+    // allocator again when a call needs more elements than it has, never because the extents merely differ, so
+    // after a call at the largest extents forward() allocates nothing (a smaller or differently shaped batch
+    // reuses the buffers; the padded positions are re-zeroed with a fill, which is not an allocation).
     void allocForForward(const LLaMAAttentionDynParams& dyn);
     void freeBuf();
 
@@ -102,7 +105,8 @@ private:
     std::unique_ptr<isp_layers::GemmEngine> gemm_;
     bool fused_attention_ = false;  // fp16 heads of 128 or 64: the fused kernel instead of steps 3-5 of the padded form
 
-    LLaMAAttentionDynParams allocated_;
+    LLaMAAttentionDynParams allocated_;   // extents of the last call (what the zeroed padding was laid out for)
+    size_t capacity_[9] = {};             // elements each buffer below holds, in their order
     T* qkv_buf_ = nullptr;      // [tokens, head_num + 2 kv_head_num, head_size]
     T* q_buf_ = nullptr;        // [batch, head_num, max_q_len, head_size]
     T* k_all_ = nullptr;        // [batch, head_num, max_k_len, head_size]

@@ -7,10 +7,17 @@
 //   ffn_weight.gateAndup     [2 * inter_size, hidden]
 //   ffn_weight.down          [hidden, inter_size]
 // and the optional biases when attn_bias is set.  loadWeights() fills them with small deterministic
-// values ("dummy" weights, as the reference's no-argument loadWeights does for performance runs);
-// loading from checkpoint files is outside this library (the reference's loader lives in
-// src/utils/weight_utils.cu).
+// values ("dummy" weights, as the reference's no-argument loadWeights does for performance runs).
+// loadWeights(weight_path, weight_type) reads the per-tensor files the reference's converter writes
+// (src/weights/llama/layer_weights.cc:45-62: raw little-endian fp32, `weight_path` + ".input_layernorm.weight.bin",
+// ".post_attention_layernorm.weight.bin", ".self_attn.qkv.weight.bin", ".self_attn.o_proj.weight.bin",
+// ".mlp.gate_up_proj.weight.bin", ".mlp.down_proj.weight.bin", and with attn_bias ".attention.wqkv.bias.bin",
+// ".attention.wo.bias.bin"), converts to T and uploads; without attn_bias the three biases are set to nullptr as
+// the reference does.  One difference: a file that is missing or shorter than its declared shape throws
+// std::runtime_error (the reference's helper prints a message and leaves the tensor as it was).
 #pragma once
+#include <string>
+
 #include "src/weights/llama/attention_weights.h"
 #include "src/weights/llama/ffn_weights.h"
 #include "src/weights/llama/norm_weights.h"
@@ -24,6 +31,7 @@ private:
     int hidden_units;
     int inter_size;
     WeightType weight_type;
+    int bit_size;
     bool attn_bias;
 
 public:
@@ -33,6 +41,8 @@ public:
     LlamaLayerWeight(const LlamaLayerWeight&) = delete;
     LlamaLayerWeight& operator=(const LlamaLayerWeight&) = delete;
     ~LlamaLayerWeight();
+
+    void loadWeights(std::string weight_path, WeightType weight_type);
 
     void loadWeights();
 

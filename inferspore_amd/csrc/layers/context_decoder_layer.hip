@@ -5,6 +5,7 @@
 #include "src/layers/decoder/context_decoder_layer.h"
 
 #include <hipblaslt/hipblaslt.h>
+#include <hipblaslt/hipblaslt-ext.hpp>
 
 #include <cmath>
 #include <cstdio>
@@ -52,12 +53,16 @@ struct LtType<half> {
 // hipBLASLt is column-major, so the call computes C^T = op(W)^T x A^T: its "A" operand is W, its
 // "B" operand is the activation, and a row-major [r, c] matrix is a column-major [c, r] one.
 //
-// The algorithm of a shape is chosen once, when the shape is first seen: the library's heuristic proposes
-// up to 128 (ISP_LAYERS_GEMM_CANDIDATES changes the number), and unless ISP_LAYERS_GEMM_AUTOTUNE=0 each is run
-// on the call's own operands (beta is 0 and no output aliases an input, so repeating the product is harmless)
-// and the fastest is kept -- the first proposal is not always the fastest on a given device, and the best of
-// 128 beats the best of 8 by 4 % of a LLaMA-2-7B layer for about 4 s at the first forward().
-// ISP_LAYERS_GEMM_VERBOSE=1 prints each choice.
+// The algorithm of a shape is chosen when the shape is first seen.  The library's heuristic proposes up to 16
+// (ISP_LAYERS_GEMM_CANDIDATES changes the number, up to 4096), and unless ISP_LAYERS_GEMM_AUTOTUNE=0 each is run on the
+// call's own operands (beta is 0 and no output aliases an input, so repeating the product is harmless) and the
+// fastest is kept -- the first proposal is not always the fastest on a given device.  That measurement is bounded:
+// it is made once per BUCKET of shapes (the row count rounded up to a multiple of 256, or to a power of two below
+// that; for the batched attention products also n and k rounded up to multiples of 64), so the ragged token counts
+// of successive prompt batches share one measurement -- a shape whose bucket has been measured takes the bucket's
+// algorithm after asking the library that it supports the exact shape -- and at most kMaxTuned buckets are ever
+// measured; later ones take the heuristic's first proposal.  The per-shape descriptor cache is emptied when it
+// reaches kMaxPlans entries.  ISP_LAYERS_GEMM_VERBOSE=1 prints each choice.
 class GemmEngine {
 public:
     explicit GemmEngine(BaseAllocator* allocator) : allocator_(allocator) {
@@ -87,7 +92,13 @@ public:
         if (m == 0 || n == 0 || batch == 0) return;
         const Key key{(int)type, m, n, k, w_is_nk ? 1 : 0, lda, ldw, ldc, batch, stride_a, stride_w, stride_c};
         auto it = plans_.find(key);
-        if (it == plans_.end()) it = plans_.emplace(key, plan(type, key, a, w, c, alpha)).first;
+        if (it == plans_.end()) {
+            if (plans_.size() >= kMaxPlans) {
+                for (auto& kv : plans_) destroy(kv.second);
+                plans_.clear();
+            }
+            it = plans_.emplace(key, plan(type, key, a, w, c, alpha)).first;
+        }
         const Plan& p = it->second;
         const float beta = 0.0f;
         ISP_LT_CHECK(hipblasLtMatmul(handle_, p.desc, &alpha, w, p.w, a, p.a, &beta, c, p.c, c, p.c, &p.algo,
@@ -97,12 +108,30 @@ public:
 private:
     static constexpr size_t kWorkspaceBytes = 32u << 20;
     static constexpr int kMaxCandidates = 4096;
+    static constexpr size_t kMaxTuned = 64;    // buckets of shapes whose algorithm is measured
+    static constexpr size_t kMaxPlans = 1024;  // exact shapes whose descriptors are kept
     using Key = std::tuple<int, int, int, int, int, int, int, int, int, long long, long long, long long>;
     struct Plan {
         hipblasLtMatmulDesc_t desc = nullptr;
         hipblasLtMatrixLayout_t w = nullptr, a = nullptr, c = nullptr;
         hipblasLtMatmulAlgo_t algo;
     };
+
+    static int bucket_rows(int v) {
+        if (v > 256) return (v + 255) / 256 * 256;
+        int p = 1;
+        while (p < v) p *= 2;
+        return p;
+    }
+    // The shape a measurement is shared by: rows rounded up; for batched products (the padded attention, whose n, k,
+    // leading dimensions and strides all follow the batch's longest query and context) those rounded or dropped too.
+    static Key bucket_of(const Key& key) {
+        int m, n, k, nk, lda, ldw, ldc, batch, t;
+        long long sa, sw, sc;
+        std::tie(t, m, n, k, nk, lda, ldw, ldc, batch, sa, sw, sc) = key;
+        if (batch > 1) return Key{t, bucket_rows(m), (n + 63) / 64 * 64, (k + 63) / 64 * 64, nk, 0, 0, 0, batch, 0, 0, 0};
+        return Key{t, bucket_rows(m), n, k, nk, lda, ldw, ldc, batch, sa, sw, sc};
+    }
 
     static void batched(hipblasLtMatrixLayout_t layout, int batch, long long stride) {
         if (batch <= 1) return;
@@ -166,7 +195,23 @@ private:
         LLM_CHECK_WITH_INFO(count > 0, "hipBLASLt offers no algorithm for a GEMM of this layer");
         int best = 0;
         float best_ms = -1.0f;
-        if (autotune_ && count > 1) {
+        const char* how = "the heuristic's first proposal";
+        const Key tuned_key = bucket_of(key);
+        auto known = tuned_.find(tuned_key);
+        if (autotune_ && known != tuned_.end()) {
+            // the bucket's measured algorithm, if the library runs it on this exact shape within the workspace
+            const float beta = 0.0f;
+            size_t need = 0;
+            hipblasLtMatmulAlgo_t algo = known->second;
+            if (hipblaslt_ext::matmulIsAlgoSupported(handle_, p.desc, &alpha, p.w, p.a, &beta, p.c, p.c, algo, need) ==
+                    HIPBLAS_STATUS_SUCCESS && need <= kWorkspaceBytes) {
+                p.algo = algo;
+                if (std::getenv("ISP_LAYERS_GEMM_VERBOSE") != nullptr)
+                    std::fprintf(stderr, "[isp_layers] GEMM m=%d n=%d k=%d batch=%d: the algorithm measured for its bucket\n", m, n, k, batch);
+                return p;
+            }
+        } else if (autotune_ && count > 1 && tuned_.size() < kMaxTuned) {
+            how = "measured";
             // a first pass over every proposal, then the four fastest again over more runs: differences of a
             // per cent or two between the leaders are inside the noise of five runs
             std::vector<std::pair<float, int>> timed;
@@ -183,10 +228,11 @@ private:
                     best = timed[j].second;
                 }
             }
+            tuned_.emplace(tuned_key, found[best].algo);
         }
         if (std::getenv("ISP_LAYERS_GEMM_VERBOSE") != nullptr)
-            std::fprintf(stderr, "[isp_layers] GEMM m=%d n=%d k=%d batch=%d: proposal %d of %d%s\n", m, n, k, batch, best, count,
-                         best_ms >= 0.0f ? (", " + std::to_string(best_ms * 1e3f) + " us").c_str() : "");
+            std::fprintf(stderr, "[isp_layers] GEMM m=%d n=%d k=%d batch=%d: proposal %d of %d (%s)%s\n", m, n, k, batch, best,
+                         count, how, best_ms >= 0.0f ? (", " + std::to_string(best_ms * 1e3f) + " us").c_str() : "");
         p.algo = found[best].algo;
         return p;
     }
@@ -203,8 +249,9 @@ private:
     hipblasLtMatmulPreference_t pref_ = nullptr;
     void* workspace_ = nullptr;
     bool autotune_ = true;
-    int candidates_ = 128;
-    std::map<Key, Plan> plans_;
+    int candidates_ = 16;
+    std::map<Key, Plan> plans_;                     // exact shapes: descriptors and the algorithm in use
+    std::map<Key, hipblasLtMatmulAlgo_t> tuned_;    // buckets of shapes: the algorithm that measured fastest
 };
 
 __device__ __forceinline__ float to_float(float x) { return x; }
@@ -460,28 +507,37 @@ size_t LlamaContextDecoderLayer<T>::workspaceBytes(const LLaMAAttentionDynParams
 
 template <typename T>
 void LlamaContextDecoderLayer<T>::allocForForward(const LLaMAAttentionDynParams& d) {
-    freeBuf();
     const size_t tokens = d.num_tokens, b = d.batch_size, q = d.max_q_len, k = d.max_k_len, hs = head_size_;
-    auto take = [this](size_t elems) {
-        return static_cast<T*>(allocator_->UnifyMalloc(nullptr, elems * sizeof(T), false));
+    bool fresh_padding = false;   // a padded buffer is new (or laid out for other extents): zero it
+    auto ensure = [this](T*& buf, size_t& capacity, size_t elems) {
+        if (elems <= capacity) return false;
+        if (buf) allocator_->UnifyFree(buf, false);
+        buf = static_cast<T*>(allocator_->UnifyMalloc(nullptr, elems * sizeof(T), false));
+        capacity = elems;
+        return true;
     };
-    qkv_buf_ = take(tokens * (head_num_ + 2 * kv_head_num_) * hs);
-    q_buf_ = take(b * head_num_ * q * hs);
+    ensure(qkv_buf_, capacity_[0], tokens * (head_num_ + 2 * kv_head_num_) * hs);
+    fresh_padding |= ensure(q_buf_, capacity_[1], b * head_num_ * q * hs);
     if (!fused_attention_) {
-        k_all_ = take(b * head_num_ * k * hs);
-        v_all_ = take(b * head_num_ * k * hs);
-        scores_ = take(b * head_num_ * q * k);
-        ctx_ = take(b * head_num_ * q * hs);
+        fresh_padding |= ensure(k_all_, capacity_[2], b * head_num_ * k * hs);
+        fresh_padding |= ensure(v_all_, capacity_[3], b * head_num_ * k * hs);
+        ensure(scores_, capacity_[4], b * head_num_ * q * k);
+        ensure(ctx_, capacity_[5], b * head_num_ * q * hs);
     }
-    ctx_packed_ = take(tokens * head_num_ * hs);
-    gate_up_ = take(tokens * 2 * inter_size_);
-    act_ = take(tokens * inter_size_);
+    ensure(ctx_packed_, capacity_[6], tokens * head_num_ * hs);
+    ensure(gate_up_, capacity_[7], tokens * 2 * inter_size_);
+    ensure(act_, capacity_[8], tokens * inter_size_);
     // padded positions of q (and the k / v rows past a sequence's context) are never written by the
-    // kernels; they only meet zero probabilities or discarded rows, but must not hold NaN patterns
-    CHECK(hipMemsetAsync(q_buf_, 0, b * head_num_ * q * hs * sizeof(T), nullptr));
-    if (!fused_attention_) {
-        CHECK(hipMemsetAsync(k_all_, 0, b * head_num_ * k * hs * sizeof(T), nullptr));
-        CHECK(hipMemsetAsync(v_all_, 0, b * head_num_ * k * hs * sizeof(T), nullptr));
+    // kernels; they only meet zero probabilities or discarded rows, but must not hold NaN patterns --
+    // nor what an earlier call with other extents left at positions that are padding now
+    const bool relaid = d.batch_size != allocated_.batch_size || d.max_q_len != allocated_.max_q_len ||
+                        (!fused_attention_ && d.max_k_len != allocated_.max_k_len);
+    if (fresh_padding || relaid) {
+        CHECK(hipMemsetAsync(q_buf_, 0, b * head_num_ * q * hs * sizeof(T), nullptr));
+        if (!fused_attention_) {
+            CHECK(hipMemsetAsync(k_all_, 0, b * head_num_ * k * hs * sizeof(T), nullptr));
+            CHECK(hipMemsetAsync(v_all_, 0, b * head_num_ * k * hs * sizeof(T), nullptr));
+        }
     }
     allocated_ = d;
 }
@@ -489,9 +545,10 @@ void LlamaContextDecoderLayer<T>::allocForForward(const LLaMAAttentionDynParams&
 template <typename T>
 void LlamaContextDecoderLayer<T>::freeBuf() {
     T** all[] = {&qkv_buf_, &q_buf_, &k_all_, &v_all_, &scores_, &ctx_, &ctx_packed_, &gate_up_, &act_};
-    for (T** p : all) {
-        if (*p) allocator_->UnifyFree(*p, false);
-        *p = nullptr;
+    for (int i = 0; i < 9; i++) {
+        if (*all[i]) allocator_->UnifyFree(*all[i], false);
+        *all[i] = nullptr;
+        capacity_[i] = 0;
     }
     allocated_ = LLaMAAttentionDynParams();
 }
@@ -528,9 +585,7 @@ void LlamaContextDecoderLayer<T>::forward(TensorMap& inputs, LlamaLayerWeight<T>
     LLM_CHECK_WITH_INFO(next_attn_norm.gamma != nullptr && weights.ffn_norm_weight.gamma != nullptr,
                         "norm weights are not loaded");
     if (tokens == 0) return;
-    if (dyn.num_tokens > allocated_.num_tokens || dyn.batch_size > allocated_.batch_size ||
-        dyn.max_q_len != allocated_.max_q_len || dyn.max_k_len != allocated_.max_k_len)
-        allocForForward(dyn);
+    allocForForward(dyn);   // grow-only: allocates only what this call needs beyond what earlier calls left
 
     const hipDataType lt = isp_layers::LtType<T>::value;
     const DataType dt = getTensorType<T>();

@@ -1,11 +1,13 @@
-// LlamaLayerWeight: device allocation in the reference's shapes and a deterministic dummy fill.
-// Follows src/weights/llama/layer_weights.cc:19-41 (constructor) and :79-120 (dummy weights) of the
-// reference; HIP runtime underneath.
+// LlamaLayerWeight: device allocation in the reference's shapes, a deterministic dummy fill and the loader of the
+// reference's per-tensor .bin files.  Follows src/weights/llama/layer_weights.cc:19-41 (constructor), :45-62 (files)
+// and :79-120 (dummy weights) of the reference; HIP runtime underneath.
 #include "src/weights/llama/layer_weights.h"
 
 #include <algorithm>
 #include <cmath>
 #include <cstdint>
+#include <cstdio>
+#include <vector>
 
 #include "src/utils/macro.h"
 
@@ -43,6 +45,24 @@ void fill(T* dst, size_t n, uint32_t tag, float scale, float shift) {
     CHECK(hipGetLastError());
 }
 
+inline void host_convert(float x, float* p) { *p = x; }
+inline void host_convert(float x, half* p) { *p = __float2half(x); }
+
+// `count` fp32 values from `filename` -> T -> device memory at dst   (src/utils/weight_utils.cu:75-140)
+template <typename T>
+void load_bin(T* dst, size_t count, const std::string& filename) {
+    LLM_CHECK_WITH_INFO(dst != nullptr, "no device memory for " + filename);
+    std::FILE* f = std::fopen(filename.c_str(), "rb");
+    LLM_CHECK_WITH_INFO(f != nullptr, "cannot open weight file " + filename);
+    std::vector<float> raw(count);
+    const size_t got = std::fread(raw.data(), sizeof(float), count, f);
+    std::fclose(f);
+    LLM_CHECK_WITH_INFO(got == count, "weight file " + filename + " is shorter than its declared shape");
+    std::vector<T> typed(count);
+    for (size_t i = 0; i < count; i++) host_convert(raw[i], &typed[i]);
+    CHECK(hipMemcpy(dst, typed.data(), count * sizeof(T), hipMemcpyHostToDevice));
+}
+
 }  // namespace
 
 template <typename T>
@@ -54,6 +74,7 @@ LlamaLayerWeight<T>::LlamaLayerWeight(int head_num, int kv_head_num, int head_si
       hidden_units(head_num * head_size),
       inter_size(inter_size),
       weight_type(weight_type),
+      bit_size(8 * (int)sizeof(T)),
       attn_bias(attn_bias) {
     const int qkv_out = (head_num + 2 * kv_head_num) * head_size;
     attn_norm_weight.gamma = device_array<T>(hidden_units);
@@ -83,6 +104,25 @@ LlamaLayerWeight<T>::~LlamaLayerWeight() {
                 ffn_weight.gateAndup.data,     ffn_weight.down.data};
     for (T* p : all)
         if (p) (void)hipFree(p);
+}
+
+template <typename T>
+void LlamaLayerWeight<T>::loadWeights(std::string weight_path, WeightType /*weight_type: unused by the reference too*/) {
+    const size_t qkv_out = (size_t)(head_num + 2 * kv_head_num) * head_size, h = (size_t)hidden_units;
+    load_bin(attn_norm_weight.gamma, h, weight_path + ".input_layernorm.weight.bin");
+    load_bin(ffn_norm_weight.gamma, h, weight_path + ".post_attention_layernorm.weight.bin");
+    load_bin(self_attn_weight.qkv.data, qkv_out * h, weight_path + ".self_attn.qkv.weight.bin");
+    load_bin(self_attn_weight.output.data, h * h, weight_path + ".self_attn.o_proj.weight.bin");
+    load_bin(ffn_weight.gateAndup.data, (size_t)2 * inter_size * h, weight_path + ".mlp.gate_up_proj.weight.bin");
+    load_bin(ffn_weight.down.data, h * inter_size, weight_path + ".mlp.down_proj.weight.bin");
+    if (attn_bias) {
+        load_bin(self_attn_weight.qkv.bias, qkv_out, weight_path + ".attention.wqkv.bias.bin");
+        load_bin(self_attn_weight.output.bias, h, weight_path + ".attention.wo.bias.bin");
+    } else {
+        self_attn_weight.qkv.bias = nullptr;
+        self_attn_weight.output.bias = nullptr;
+        ffn_weight.down.bias = nullptr;
+    }
 }
 
 template <typename T>

@@ -74,6 +74,9 @@ __device__ __forceinline__ void norm_rows_body(T* residual, T* out, const T* bia
     T* out_row = out + base;
     T* rsd_row = residual + base;  // dereferenced only when has_res
 
+    // the small operands' addresses are fetched with the other arguments at kernel entry (left alone, the
+    // compiler fetches the gamma pointer only where it is first used: a scalar round trip behind the row's arrival)
+    asm volatile("" : : "s"(gamma), "s"(bias));
     vec16 vo[NV], vr[NV];
     bool ok[NV];
 #pragma unroll

@@ -5,7 +5,10 @@
 // case checks, inside the program, that two turns through the KV cache reproduce one long prefill.
 //
 //   test_context_layer <f32|f16> <directory> [head_num kv_head_num head_size inter_size]
+#include <algorithm>
+#include <cmath>
 #include <cstdio>
+#include <cstring>
 #include <memory>
 #include <numeric>
 #include <string>
@@ -335,6 +338,102 @@ static int run(const std::string& dir, int head_num, int kv_heads, int head_size
             CHECK(hipFree(d_hl));
             CHECK(hipFree(d_il));
             CHECK(hipFree(d_cl));
+        }
+    }
+
+    // ---- case 5: weights written as the reference's per-tensor fp32 files load back to the same bits
+    {
+        const std::string prefix = dir + "/model.layers.0";
+        const int qkv_n = (head_num + 2 * kv_heads) * head_size;
+        auto write = [&](const char* suffix, const T* device, size_t n) { dump<T>(dir, (std::string("model.layers.0") + suffix).c_str(), device, n); };
+        // dump() appends ".bin", the names are the reference's (src/weights/llama/layer_weights.cc:47-57)
+        write(".input_layernorm.weight", w.attn_norm_weight.gamma, hidden);
+        write(".post_attention_layernorm.weight", w.ffn_norm_weight.gamma, hidden);
+        write(".self_attn.qkv.weight", w.self_attn_weight.qkv.data, (size_t)qkv_n * hidden);
+        write(".self_attn.o_proj.weight", w.self_attn_weight.output.data, (size_t)hidden * hidden);
+        write(".mlp.gate_up_proj.weight", w.ffn_weight.gateAndup.data, (size_t)2 * inter * hidden);
+        write(".mlp.down_proj.weight", w.ffn_weight.down.data, (size_t)hidden * inter);
+        write(".attention.wqkv.bias", w.self_attn_weight.qkv.bias, qkv_n);
+        write(".attention.wo.bias", w.self_attn_weight.output.bias, hidden);
+        auto same = [&](const T* a, const T* b, size_t n) {
+            auto x = to_host((const S*)a, n), y = to_host((const S*)b, n);
+            return std::memcmp(x.data(), y.data(), n * sizeof(S)) == 0;
+        };
+        LlamaLayerWeight<T> loaded(head_num, kv_heads, head_size, inter, getWeightType<T>(), /*attn_bias=*/true);
+        loaded.loadWeights(prefix, getWeightType<T>());
+        EXPECT(same(loaded.attn_norm_weight.gamma, w.attn_norm_weight.gamma, hidden) &&
+                   same(loaded.ffn_norm_weight.gamma, w.ffn_norm_weight.gamma, hidden) &&
+                   same(loaded.self_attn_weight.qkv.data, w.self_attn_weight.qkv.data, (size_t)qkv_n * hidden) &&
+                   same(loaded.self_attn_weight.output.data, w.self_attn_weight.output.data, (size_t)hidden * hidden) &&
+                   same(loaded.ffn_weight.gateAndup.data, w.ffn_weight.gateAndup.data, (size_t)2 * inter * hidden) &&
+                   same(loaded.ffn_weight.down.data, w.ffn_weight.down.data, (size_t)hidden * inter) &&
+                   same(loaded.self_attn_weight.qkv.bias, w.self_attn_weight.qkv.bias, qkv_n) &&
+                   same(loaded.self_attn_weight.output.bias, w.self_attn_weight.output.bias, hidden),
+               "weights loaded from files differ from the ones written");
+        LlamaLayerWeight<T> no_bias(head_num, kv_heads, head_size, inter, getWeightType<T>(), /*attn_bias=*/false);
+        no_bias.loadWeights(prefix, getWeightType<T>());
+        EXPECT(no_bias.self_attn_weight.qkv.bias == nullptr && no_bias.self_attn_weight.output.bias == nullptr &&
+                   no_bias.ffn_weight.down.bias == nullptr,
+               "without attn_bias the loader must leave every bias null");
+        EXPECT(same(no_bias.ffn_weight.down.data, w.ffn_weight.down.data, (size_t)hidden * inter), "down weight without bias");
+        EXPECT(throws([&] { loaded.loadWeights(dir + "/no.such.layer", getWeightType<T>()); }), "a missing weight file must throw");
+    }
+
+    // ---- case 6: after a call at the largest extents the layer takes nothing more from the allocator
+    {
+        struct Counting : HipAllocator {
+            int mallocs = 0;
+            void* UnifyMalloc(void* ptr, size_t size, bool is_host = false) override {
+                mallocs++;
+                return HipAllocator::UnifyMalloc(ptr, size, is_host);
+            }
+        } counting;
+        {
+            LlamaContextDecoderLayer<T> fresh(head_num, kv_heads, head_size, inter, params, 1e-5f, &counting);
+            const size_t one = (size_t)3 * kv_heads * max_seq * head_size;
+            T* kc6 = (T*)to_device(std::vector<S>(one));
+            T* vc6 = (T*)to_device(std::vector<S>(one));
+            auto call = [&](const std::vector<int>& l, const std::vector<int>& h, std::vector<S>& next_out) {
+                Batch<T> b6(l, h, *std::max_element(l.begin(), l.end()));
+                std::vector<S> part(rows.begin(), rows.begin() + (size_t)b6.tokens * hidden);
+                T* r = (T*)to_device(part);
+                T* nrm = (T*)to_device(std::vector<S>(part.size()));
+                T* o = (T*)to_device(std::vector<S>(part.size()));
+                run_layer(fresh, w, next, b6, r, nrm, o, kc6, vc6, 1, kv_heads, max_seq, head_size, hidden, 0);
+                next_out = to_host((S*)o, part.size());
+                CHECK(hipFree(r));
+                CHECK(hipFree(nrm));
+                CHECK(hipFree(o));
+            };
+            std::vector<S> big, small_after, small_alone;
+            call({16, 5, 11}, {0, 0, 0}, big);
+            const int after_first = counting.mallocs;
+            EXPECT(after_first > 0, "the first call must allocate the layer's buffers");
+            call({4, 9}, {0, 0}, small_after);          // fewer sequences, shorter, other padded extents
+            call({16, 5, 11}, {0, 0, 0}, big);
+            call({1, 1, 1}, {7, 2, 9}, small_after);    // a decode-shaped call: one token each, longer contexts
+            call({4, 9}, {0, 0}, small_after);
+            EXPECT(counting.mallocs == after_first, "later, smaller calls allocated %d more buffers", counting.mallocs - after_first);
+            // ... and a buffer that held a larger batch gives the results of a layer that never saw one
+            LlamaContextDecoderLayer<T> clean(head_num, kv_heads, head_size, inter, params, 1e-5f, &allocator);
+            T* kc7 = (T*)to_device(std::vector<S>(one));
+            T* vc7 = (T*)to_device(std::vector<S>(one));
+            {
+                Batch<T> b7({4, 9}, {0, 0}, 9);
+                std::vector<S> part(rows.begin(), rows.begin() + (size_t)b7.tokens * hidden);
+                T* r = (T*)to_device(part);
+                T* nrm = (T*)to_device(std::vector<S>(part.size()));
+                T* o = (T*)to_device(std::vector<S>(part.size()));
+                run_layer(clean, w, next, b7, r, nrm, o, kc7, vc7, 1, kv_heads, max_seq, head_size, hidden, 0);
+                small_alone = to_host((S*)o, part.size());
+            }
+            double err = 0, scale = 0;
+            for (size_t i = 0; i < small_alone.size(); i++) {
+                scale = std::max(scale, std::fabs((double)Host<T>::from(small_alone[i])));
+                err = std::max(err, std::fabs((double)Host<T>::from(small_alone[i]) - Host<T>::from(small_after[i])));
+            }
+            // each layer object measures its GEMM algorithms for itself: allow for another summation order
+            EXPECT(err <= (std::is_same<T, float>::value ? 3e-4 : 3e-2) * scale, "reused buffers change the result by %g (scale %g)", err, scale);
         }
     }
 
