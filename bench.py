@@ -59,6 +59,10 @@ def parse():
     ap.add_argument("--copy-curve", action="store_true",
                     help="instead of the workloads, time the plain copy at 8 MiB .. 1 GiB of traffic per launch "
                          "(the practical ceiling as a function of launch size) and print it as one JSON line")
+    ap.add_argument("--gather-locality", action="store_true",
+                    help="instead of the workloads, time the embedding gather with ids in random runs of 1, 2, 4, 8, 32 "
+                         "consecutive table rows and with the rows in order, beside a copy of equal bytes: how much of "
+                         "the gather's distance to the copy is the randomness of its rows (one JSON line)")
     ap.add_argument("--cpu-seconds", type=float, default=20.0, help="budget of the CPU baseline leg")
     return ap.parse_args()
 
@@ -190,17 +194,27 @@ def make_workloads(torch, lib, stream_handle, rotate):
         w.config = {"tokens": tokens, "hidden": hidden}
         return w
 
-    def embedding(tdtype=torch.float16):
+    def embedding(tdtype=torch.float16, id_run=1):
+        """id_run: 1 = independent random ids (the configuration); n > 1 = random runs of n consecutive table
+        rows; 0 = the table rows in order (what a copy reads)."""
         w = Workload()
         tokens, hidden, vocab = 8192, 4096, 32000
         es = 2 if tdtype == torch.float16 else 4
         sfx = "f16" if es == 2 else "f32"
         w.name, w.dtype, w.tokens = "embedding_%s_8192x4096_v32000" % sfx, sfx, tokens
+        if id_run != 1:
+            w.name += "_runs_of_%d" % id_run
         w.kernel = "isp::gather_chunks_vec<2>"
         w.bytes_per_launch = 2 * tokens * hidden * es + tokens * 4
         table = (0.02 * torch.randn((vocab, hidden), device=dev)).to(tdtype)
         R = w.sets_for(tokens * hidden * es, rotate)
-        ids = [torch.randint(0, vocab, (tokens,), device=dev, dtype=torch.int32) for _ in range(R)]
+        if id_run == 1:
+            ids = [torch.randint(0, vocab, (tokens,), device=dev, dtype=torch.int32) for _ in range(R)]
+        elif id_run == 0:
+            ids = [((torch.arange(tokens, device=dev) + j * tokens) % vocab).to(torch.int32) for j in range(R)]
+        else:
+            ids = [(torch.randint(0, vocab - id_run, (tokens // id_run,), device=dev).repeat_interleave(id_run) +
+                    torch.arange(tokens, device=dev) % id_run).to(torch.int32) for _ in range(R)]
         outs = [torch.empty((tokens, hidden), device=dev, dtype=tdtype) for _ in range(R)]
         w.keep = (table, ids, outs)
         w.bind(getattr(lib, "isp_embedding_" + sfx), [(ids[j].data_ptr(), outs[j].data_ptr(), table.data_ptr(), tokens, hidden,
@@ -218,19 +232,22 @@ def make_workloads(torch, lib, stream_handle, rotate):
         assert lib.isp_cal_padding_offset(po.data_ptr(), cum.data_ptr(), lens_d.data_ptr(), batch, seq, st) == 0
         return batch, seq, int(lens.sum()), lens_d, po
 
-    def qkv(tdtype=torch.float16, hn=32, kvn=32, hs=128, tag=""):
+    def qkv(tdtype=torch.float16, hn=32, kvn=32, hs=128, tag="", with_bias=True):
         w = Workload()
         es = 2 if tdtype == torch.float16 else 4
         sfx = "f16" if es == 2 else "f32"
         batch, seq, tokens, lens_d, po = padded_batch()
         w.name, w.dtype, w.tokens = "qkv_bias_rope_transpose_%s_b8_s512%s" % (sfx, tag), sfx, tokens
+        flag = "true" if with_bias else "false"
         if es == 2 and hs == 128 and hn % 32 == 0 and kvn % 32 == 0:
-            w.kernel = "isp::qkv_rope_lean_f16<2, true, false>"
+            w.kernel = "isp::qkv_rope_lean_f16<2, %s, false>" % flag
         else:
-            w.kernel = "isp::qkv_rope_wave<%s, %d, 2, 4, true>" % ("__half" if es == 2 else "float", hs)
-        w.bytes_per_launch = tokens * (2 * (hn + 2 * kvn) * hs * es + 4) + (hn + 2 * kvn) * hs * es + 2 * batch * 4
+            w.kernel = "isp::qkv_rope_wave<%s, %d, 2, 4, %s>" % ("__half" if es == 2 else "float", hs, flag)
+        w.bytes_per_launch = tokens * (2 * (hn + 2 * kvn) * hs * es + 4) + 2 * batch * 4
+        if with_bias:
+            w.bytes_per_launch += (hn + 2 * kvn) * hs * es
         hist = torch.zeros(batch, device=dev, dtype=torch.int32)
-        bias = (0.02 * torch.randn((hn + 2 * kvn) * hs, device=dev)).to(tdtype)
+        bias = (0.02 * torch.randn((hn + 2 * kvn) * hs, device=dev)).to(tdtype) if with_bias else None
         set_bytes = tokens * (hn + 2 * kvn) * hs * es + batch * (hn + 2 * kvn) * seq * hs * es
         R = w.sets_for(set_bytes, rotate)
         ins = [torch.randn((tokens, hn + 2 * kvn, hs), device=dev).to(tdtype) for _ in range(R)]
@@ -239,8 +256,8 @@ def make_workloads(torch, lib, stream_handle, rotate):
         w.keep = (lens_d, po, hist, bias, ins, outs)
         w.bind(getattr(lib, "isp_qkv_bias_rope_transpose_" + sfx),
                [(outs[j][0].data_ptr(), outs[j][1].data_ptr(), outs[j][2].data_ptr(), ins[j].data_ptr(),
-                 bias.data_ptr(), po.data_ptr(), hist.data_ptr(), lens_d.data_ptr(), batch, seq, tokens, hn, kvn, hs,
-                 hs, 10000.0, 2048, 0, st) for j in range(R)])
+                 bias.data_ptr() if with_bias else None, po.data_ptr(), hist.data_ptr(), lens_d.data_ptr(), batch, seq,
+                 tokens, hn, kvn, hs, hs, 10000.0, 2048, 0, st) for j in range(R)])
         w.reset = lambda: None
         w.config = {"batch": batch, "max_seq": seq, "valid_tokens": tokens, "heads": "%dq/%dkv" % (hn, kvn),
                     "head_dim": hs}
@@ -369,6 +386,9 @@ def make_workloads(torch, lib, stream_handle, rotate):
     def copy(nbytes):
         return make_copy_workload(torch, lib, st, nbytes, rotate)
 
+    if rotate == "gather-locality":
+        return [("embedding_f16_8192x4096_v32000" + ("_runs_of_%d" % n if n != 1 else ""),
+                 (lambda n=n: embedding(id_run=n))) for n in (1, 2, 4, 8, 32, 0)] + [("calibration_copy_128MiB_traffic", lambda: copy(64 << 20))]
     table = [
         (HEADLINE, lambda: norm(HEADLINE, 2048, 4096, torch.float16, True)),
         # the same kernel at the row counts a prefill layer hands it (the ragged batch's 2977 valid tokens; 4096)
@@ -380,6 +400,8 @@ def make_workloads(torch, lib, stream_handle, rotate):
         ("rmsnorm_f32_16384x4096", lambda: norm("rmsnorm_f32_16384x4096", 16384, 4096, torch.float32, False)),
         ("embedding_f16_8192x4096_v32000", embedding),
         ("qkv_bias_rope_transpose_f16_b8_s512", qkv),
+        # the same step as LLaMA runs it: its projections have no bias (layer_weights.cc:58-62 sets the pointers to null)
+        ("qkv_bias_rope_transpose_f16_b8_s512_no_bias", lambda: qkv(tag="_no_bias", with_bias=False)),
         ("qkv_bias_rope_transpose_append_f16_b8_s512_S1024", lambda: qkv_append(True)),
         ("qkv_bias_rope_transpose_then_concat_kv_f16_b8_s512_S1024", lambda: qkv_append(False)),
         ("swiglu_f16_prefill_8192x11008", lambda: swiglu(8192, "prefill")),
@@ -394,6 +416,8 @@ def make_workloads(torch, lib, stream_handle, rotate):
         ("embedding_f32_8192x4096_v32000", lambda: embedding(torch.float32)),
         ("qkv_bias_rope_transpose_f32_b8_s512", lambda: qkv(torch.float32)),
         ("swiglu_f32_prefill_8192x11008", lambda: swiglu(8192, "prefill", torch.float32)),
+        ("calibration_copy_2MiB_traffic", lambda: copy(1 << 20)),
+        ("calibration_copy_16MiB_traffic", lambda: copy(8 << 20)),
         ("calibration_copy_64MiB_traffic", lambda: copy(32 << 20)),
         ("calibration_copy_512MiB_traffic", lambda: copy(256 << 20)),
     ]
@@ -993,6 +1017,14 @@ def main():
                           "points": points, "fit": {"fixed_us": my - slope * mx, "asymptotic_GBps": 1e-3 / slope}}))
         return
 
+    if a.gather_locality:
+        pts = run_all("gather-locality")
+        print(json.dumps({"metric": "embedding gather vs locality of the token ids (8192 ids, 32000 x 4096 fp16 table)",
+                          "unit": "us per launch",
+                          "points": {r["workload"]: {"us": round(r["ms_per_launch_events"] * 1e3, 3),
+                                                     "GBps": round(r["GBps"], 1)} for r in pts}}))
+        return
+
     results = run_all(True)
     head = results[0]
     # The practical ceiling of this device for a read+write stream, from the two plain copies of
@@ -1006,9 +1038,26 @@ def main():
             c_big["ms_per_launch_events"] - c_small["ms_per_launch_events"])          # bytes per ms
         fixed = c_small["ms_per_launch_events"] - c_small["algorithmic_bytes"] / rate  # ms
         copy_model = {"fixed_us": round(fixed * 1e3, 3), "asymptotic_GBps": round(rate / 1e6, 1),
-                      "form": "copy_time = fixed_us + bytes / asymptotic rate"}
+                      "form": "copy_time = fixed_us + bytes / asymptotic rate from 64 MiB of traffic up; below that, "
+                              "interpolated between the copies measured at 2, 16 and 64 MiB of traffic (a launch "
+                              "of a few MiB does not ramp up to the asymptotic rate)"}
+        # measured copy points (bytes, ms), ascending: the model passes through every one of them
+        points = sorted((r["algorithmic_bytes"], r["ms_per_launch_events"]) for r in results
+                        if r["workload"].startswith("calibration_copy_"))
+        copy_model["measured_us"] = {"%dMiB" % (b >> 20): round(t * 1e3, 3) for b, t in points}
+
+        def copy_time(nbytes):
+            if nbytes >= points[-2][0] or len(points) < 3:
+                return fixed + nbytes / rate
+            if nbytes <= points[0][0]:
+                return points[0][1]   # the floor: a smaller launch is not faster
+            for (b0, t0), (b1, t1) in zip(points, points[1:]):
+                if nbytes <= b1:
+                    return t0 + (t1 - t0) * (nbytes - b0) / (b1 - b0)
+            return fixed + nbytes / rate
+
         for r in results:
-            t = fixed + r["algorithmic_bytes"] / rate
+            t = copy_time(r["algorithmic_bytes"])
             r["copy_model_ms"] = t
             r["vs_copy"] = t / r["ms_per_launch_events"]
     config = {"workload": head["workload"], "storage_dtype": "f16", "tokens_per_s": head["tokens_per_s"],

@@ -179,7 +179,7 @@ int isp_swiglu_f16(const void* in, void* out, int tokens, int inter, isp_stream_
 
 /*
  * Decode-phase RoPE, in place: rotate-half on the q and k heads of packed rows
- * [batch, head_num + 2 kv_head_num, head_size] at timestep step - 1.
+ * [batch, head_num + 2 kv_head_num, head_size] at timestep step - 1 (step >= 1).
  * Replaces launchRoPE<T> (src/kernels/qkv_bias_and_RoPE.h:22-25, .cu:352-434; the reference's fp16
  * body is empty and its launcher only accepts batch 1, 32+32+32 heads of 128).
  */
@@ -197,6 +197,10 @@ int isp_rope_decode_f16(void* qkv, int batch, int head_num, int kv_head_num, int
  * launchConcatKVCache<T> with a one-token query (src/kernels/concat_past_kv.cu:7-113), whose results
  * it reproduces bit for bit; each of the two is launch-bound alone.  The reference has no fused form
  * outside its attention kernel (src/kernels/fused_decoder_self_attention.cu:162-200).
+ * The one timestep step - 1 for the whole batch is the reference's launchRoPE (which only accepts batch 1);
+ * it agrees with the row the append writes only where history_length[b] == step - 1.  For a batch whose
+ * sequences have different histories pass step = 0: every sequence is then rotated at its own
+ * history_length[b], the position its row is appended at (= the prefill kernel on one-token sequences).
  */
 int isp_rope_decode_append_f32(void* qkv, const void* bias, void* k_cache, void* v_cache, int layer,
                                int max_seq_len, const int32_t* history_length, int batch,

@@ -53,7 +53,11 @@ class GemmEngine;  // hipBLASLt handle, workspace and per-shape algorithm cache
 // positions <= history_length[b] + q and < context_length[b] -- and exactly zero elsewhere; rows of padded
 // queries (q >= input_length[b]) become zero.  The mask is computed from the three [batch] length arrays
 // instead of being read from a [batch, q, k] tensor (src/kernels/build_casual_mask.cu:5-42,
-// attn_softmax_kernel.cu:50-125).  Instantiated for float and half.
+// attn_softmax_kernel.cu:50-125).  One deliberate departure when a sequence has history: the reference's mask
+// also requires k >= context length - query length (build_casual_mask.cu:36), which hides every history key
+// (its own comment calls that the mask without multi-turn support and draws the other one); here, and in the
+// fused kernel below, a query attends to the history as well.  Identical when history_length = 0.
+// Instantiated for float and half.
 template <typename T>
 void launch_masked_scaled_softmax(T* scores, const int* history_length, const int* input_length,
                                   const int* context_length, int batch, int head_num, int max_q_len,

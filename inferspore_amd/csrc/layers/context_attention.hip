@@ -6,7 +6,11 @@
 // registers, and key tiles behind the causal diagonal are not visited.
 //
 // The mask is the one of the layer's softmax: query q of sequence b sees the keys at positions
-// < min(history_length[b] + q + 1, context_length[b], max_k_len)  (src/kernels/build_casual_mask.cu:5-42).
+// < min(history_length[b] + q + 1, context_length[b], max_k_len).  A deliberate departure from the reference when a
+// sequence has history: its mask (src/kernels/build_casual_mask.cu:36) additionally requires k >= context length -
+// query length, which hides every history key -- the comment above that line calls it the mask that does not support
+// multi-turn dialogue and draws the one that does, which is the one computed here.  With history_length = 0 the two
+// are the same mask.
 //
 // Matrix cores: v_mfma_f32_32x32x16_f16.  A wavefront owns 32 queries.  It computes the TRANSPOSED scores
 // S^T[key, query] = K x Q^T, so that a lane's 16 accumulators of a 32 x 32 block all belong to one query

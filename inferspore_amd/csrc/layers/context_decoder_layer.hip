@@ -278,7 +278,9 @@ __device__ __forceinline__ float block_reduce(float v, bool take_max, float* sha
 // < context_length[b] -- and zero elsewhere; rows of padded queries (q >= input_length[b]) become zero.
 // What the reference does with launchBuildCausalMasks + launchScaleMaskAndSoftmax
 // (src/kernels/build_casual_mask.cu:5-42, attn_softmax_kernel.cu:50-125), with the mask computed
-// from the lengths instead of read from a [batch, q, k] tensor.  fp32 arithmetic.
+// from the lengths instead of read from a [batch, q, k] tensor -- and with the history keys visible,
+// which the reference's mask hides (build_casual_mask.cu:36: k >= klen - qlen; see the header).
+// fp32 arithmetic.
 template <typename T>
 __global__ __launch_bounds__(256) void masked_scaled_softmax(T* scores, const int* history_length,
                                                              const int* input_length,

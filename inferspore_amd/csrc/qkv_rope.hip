@@ -694,10 +694,12 @@ __global__ __launch_bounds__(kBlock) void rope_decode_wave(T* __restrict__ qkv, 
             bhi = load16(ex.bias + (size_t)h * HS + HALF + g * VEC);
         }
     }
+    // timestep < 0: each sequence at its own position history_length[b] (a batch of ragged histories)
+    const int t = timestep >= 0 ? timestep : read_only_i32(ex.history_length, b);
     __shared__ float2 cs[WAVES][HALF];
     if (lane < HALF) {
         float2 coef = make_float2(1.0f, 0.0f);
-        if (lane < half_rot) coef = rope_coefficients(timestep, tab.div[lane]);
+        if (lane < half_rot) coef = rope_coefficients(t, tab.div[lane]);
         cs[wave][lane] = coef;
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -758,6 +760,7 @@ __global__ __launch_bounds__(kBlock) void rope_decode_generic(T* qkv, int head_n
     // without extras only the rotated pairs are touched; with them every pair of every covered head
     const int per_head = extras ? half : half_rot;
     const int pairs = covered * per_head;
+    const int t = timestep >= 0 ? timestep : read_only_i32(ex.history_length, b);
     long long cache_row = -1;
     if (ex.k_cache) {
         cache_row = read_only_i32(ex.history_length, b);
@@ -774,7 +777,7 @@ __global__ __launch_bounds__(kBlock) void rope_decode_generic(T* qkv, int head_n
         }
         float y0 = x0, y1 = x1;
         if (!is_v && d < half_rot) {
-            const float2 coef = rope_coefficients(timestep, tab.div[d]);
+            const float2 coef = rope_coefficients(t, tab.div[d]);
             rotate_pair(coef.x, coef.y, x0, x1, y0, y1);
         }
         const T o0 = Elem<T>::from_f32(y0), o1 = Elem<T>::from_f32(y1);
@@ -836,7 +839,12 @@ static int rope_decode(void* qkv_, int batch, int head_num, int kv_head_num, int
     }
     RopeDivisors tab;
     fill_divisors(tab, rot, base);
-    const int timestep = step - 1;  // qkv_bias_and_RoPE.cu:380
+    // step >= 1: every sequence at timestep step - 1 (qkv_bias_and_RoPE.cu:380).  step == 0 (the fused decode step
+    // only): each sequence at its own history_length[b], the position its k / v row is appended at -- a batch whose
+    // sequences have different histories.  The kernels take that as a negative timestep.
+    if (step == 0) ISP_REQUIRE_PTR(history_length);
+    if (step < 0) return ISP_ERR_BAD_SHAPE;
+    const int timestep = step - 1;
     const int half_rot = rot / 2;
     const int covered = head_num + kv_head_num + ((ex.bias || ex.k_cache) ? kv_head_num : 0);
     dim3 block(kBlock);

@@ -225,7 +225,8 @@ def rope_decode_and_append(qkv_buf, qkv_bias, k_cache, v_cache, layer_id, histor
     """One decode step's bias + rotate-half RoPE + KV-cache append in a single launch: in place on qkv_buf
     [batch, head_num + 2 kv_head_num, head_size] at timestep step - 1 (as launchRoPE), and the rotated k row and
     the v row of sequence b go to cache[layer][b, head, history_length[b], :] (as launchConcatKVCache with one
-    query token).  qkv_bias may be None."""
+    query token).  qkv_bias may be None.  step = 0: every sequence is rotated at its own history_length[b] instead
+    (a batch whose sequences have different histories)."""
     _same_dtype(qkv_buf, qkv_bias, k_cache, v_cache)
     _int32(history_length)
     _expect(qkv_buf.dim() == 3, "qkv_buf must be [batch, heads, head_size]")

@@ -187,3 +187,43 @@ def test_decode_step_with_bias_equals_the_prefill_kernel(isp, oracle, dtype, hn,
             assert_f32_close(got.cpu().numpy()[:, :, 0], exp[:, :, 0], "decode with bias", scale=rad[:, sl] + 1e-30)
         else:
             assert_f16_close(got.cpu().numpy()[:, :, 0], exp[:, :, 0], "decode with bias", magnitude=rad[:, sl])
+
+
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+@pytest.mark.parametrize("hn,kvn,hs,rot,with_bias", [(32, 32, 128, 128, False), (8, 2, 128, 64, True), (4, 4, 64, 64, True),
+                                                     (3, 1, 16, 16, False)])
+def test_decode_step_with_ragged_histories_rotates_each_sequence_at_its_own_position(isp, dtype, hn, kvn, hs, rot, with_bias):
+    """step = 0: sequence b is rotated at history_length[b], where its row is appended -- the prefill kernel on
+    one-token sequences with those histories, bit for bit.  (With one step for the whole batch the rotation and the
+    cache row only agree where history_length[b] == step - 1.)"""
+    say("ragged decode step %s hn=%d kvn=%d hs=%d rot=%d bias=%s" % (dtype.__name__, hn, kvn, hs, rot, with_bias))
+    batch, max_seq = 6, 256
+    r = np.random.default_rng(hs * 3 + hn)
+    td = NP2T[dtype]
+    x = r.standard_normal((batch, hn + 2 * kvn, hs), dtype=np.float32).astype(dtype)
+    bias = (0.02 * r.standard_normal((hn + 2 * kvn) * hs)).astype(dtype) if with_bias else None
+    hist = torch.tensor([0, 5, 200, 17, 255, 63], dtype=torch.int32, device="cuda")
+    ones = torch.ones(batch, dtype=torch.int32, device="cuda")
+    zeros = torch.zeros(batch, dtype=torch.int32, device="cuda")
+    q = torch.zeros((batch, hn, 1, hs), dtype=td, device="cuda")
+    kc1 = torch.full((1, batch, kvn, max_seq, hs), SENTINEL, dtype=td, device="cuda")
+    vc1 = kc1.clone()
+    isp.add_fused_qkv_bias_transpose_rope_and_append(q, None, None, kc1, vc1, 0, dev(x), dev(bias), zeros, hist, ones, rot,
+                                                     10000.0)
+    y = dev(x)
+    kc2, vc2 = torch.full_like(kc1, SENTINEL), torch.full_like(kc1, SENTINEL)
+    isp.rope_decode_and_append(y, dev(bias), kc2, vc2, 0, hist, 0, hn, rot, 10000.0)
+    torch.cuda.synchronize()
+    assert torch.equal(y[:, :hn], q[:, :, 0])
+    assert torch.equal(kc1, kc2) and torch.equal(vc1, vc2)
+    for b, h in enumerate(hist.tolist()):
+        assert torch.equal(y[b, hn:hn + kvn], kc2[0, b, :, h])
+    # one step for everybody is a different operation on this batch: it must not give the same rows
+    y1 = dev(x)
+    kc3, vc3 = torch.full_like(kc1, SENTINEL), torch.full_like(kc1, SENTINEL)
+    isp.rope_decode_and_append(y1, dev(bias), kc3, vc3, 0, hist, 6, hn, rot, 10000.0)
+    torch.cuda.synchronize()
+    assert torch.equal(y1[1], y[1]) and not torch.equal(y1[2, :hn + kvn], y[2, :hn + kvn])
+    # the plain decode RoPE has no per-sequence positions: step 0 is rejected there
+    with pytest.raises(RuntimeError):
+        isp.rope(dev(x), 0, hn, rot, 10000.0)
