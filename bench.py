@@ -154,13 +154,13 @@ def make_workloads(torch, lib, stream_handle, rotate):
     dev = "cuda"
     st = stream_handle
 
-    def norm(name, tokens, hidden, tdtype, fused):
+    def norm(name, tokens, hidden, tdtype, fused, with_bias=True):
         w = Workload()
         es = 2 if tdtype == torch.float16 else 4
         sfx = "f16" if es == 2 else "f32"
         w.name, w.dtype, w.tokens = name, sfx, tokens
         if fused:
-            w.bytes_per_launch = 4 * tokens * hidden * es + 2 * hidden * es
+            w.bytes_per_launch = 4 * tokens * hidden * es + (2 if with_bias else 1) * hidden * es
             set_bytes = 2 * tokens * hidden * es
         else:
             w.bytes_per_launch = 2 * tokens * hidden * es + hidden * es
@@ -170,14 +170,14 @@ def make_workloads(torch, lib, stream_handle, rotate):
         # land on separately mapped pages, and launch-bound kernels then time up to 2x slower
         outs = list(torch.empty((R, tokens, hidden), device=dev, dtype=tdtype).normal_().unbind(0))
         ress = list(torch.empty((R, tokens, hidden), device=dev, dtype=tdtype).normal_().unbind(0)) if fused else None
-        bias = (0.02 * torch.randn(hidden, device=dev)).to(tdtype) if fused else None
+        bias = (0.02 * torch.randn(hidden, device=dev)).to(tdtype) if fused and with_bias else None
         gamma = (0.5 + torch.rand(hidden, device=dev)).to(tdtype)
         w.keep = (outs, ress, bias, gamma)
         w.kernel = norm_kernel_name(lib, es, tokens, hidden, fused)
         if fused:
             fn = getattr(lib, "isp_fused_add_bias_residual_rmsnorm_" + sfx)
-            w.bind(fn, [(ress[j].data_ptr(), outs[j].data_ptr(), bias.data_ptr(), gamma.data_ptr(), 1e-5, tokens,
-                         hidden, 0, st) for j in range(R)])
+            w.bind(fn, [(ress[j].data_ptr(), outs[j].data_ptr(), bias.data_ptr() if with_bias else None, gamma.data_ptr(),
+                         1e-5, tokens, hidden, 0, st) for j in range(R)])
         else:
             fn = getattr(lib, "isp_rmsnorm_" + sfx)
             w.bind(fn, [(outs[j].data_ptr(), gamma.data_ptr(), 1e-5, tokens, hidden, st) for j in range(R)])
@@ -396,6 +396,11 @@ def make_workloads(torch, lib, stream_handle, rotate):
          lambda: norm("fused_add_bias_residual_rmsnorm_f16_2977x4096", 2977, 4096, torch.float16, True)),
         ("fused_add_bias_residual_rmsnorm_f16_4096x4096",
          lambda: norm("fused_add_bias_residual_rmsnorm_f16_4096x4096", 4096, 4096, torch.float16, True)),
+        # ... and as LLaMA calls it: a residual but no bias (its projections have none, layer_weights.cc:58-62)
+        ("fused_add_residual_rmsnorm_f16_2048x4096_no_bias",
+         lambda: norm("fused_add_residual_rmsnorm_f16_2048x4096_no_bias", 2048, 4096, torch.float16, True, False)),
+        ("fused_add_residual_rmsnorm_f16_2977x4096_no_bias",
+         lambda: norm("fused_add_residual_rmsnorm_f16_2977x4096_no_bias", 2977, 4096, torch.float16, True, False)),
         ("rmsnorm_f32_64x4096", lambda: norm("rmsnorm_f32_64x4096", 64, 4096, torch.float32, False)),
         ("rmsnorm_f32_16384x4096", lambda: norm("rmsnorm_f32_16384x4096", 16384, 4096, torch.float32, False)),
         ("embedding_f16_8192x4096_v32000", embedding),

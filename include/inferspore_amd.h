@@ -308,7 +308,10 @@ typedef enum isp_tuning_knob {
                                         workgroup when a row needs fewer); 0 = automatic */
     ISP_TUNE_NORM_ORDER = 9,         /* 2 = streaming (each vector processed, and the residual stored, as it
                                         arrives); 0, 1 = read everything, then write everything (default);
-                                        3 = as 0, but launches of a few rows also take the general kernel */
+                                        3 = as 0, but launches of a few rows also take the general kernel;
+                                        4 / 5 = as 0, but a call with a residual and no bias never / always waits
+                                        for a gamma vector where the bias vector would arrive (by default it does
+                                        where the launch is one round of waves reading more than 24 MiB) */
     ISP_TUNE_MOVER_BLOCK_THREADS = 10, /* KV append / broadcast: 256, 512 or 1024 threads per workgroup */
     ISP_TUNE_COUNT = 11
 } isp_tuning_knob;

@@ -48,6 +48,17 @@ __device__ __forceinline__ float tree_sum(const float* p) {
 // knob): with several rounds of waves it measured within 1 % of the order above for 16-bit rows and
 // plain RMSNorm, and 8-12 % slower for 32-bit rows with a residual.  Same bits under both.
 constexpr unsigned kNormStreamingOrder = 0x80000000u;
+// Step 3 is more than a way to fetch the bias: the cache round trip it puts between the arrival of a wave's rows
+// and its first store is what keeps the early waves' stores out of the late waves' reads.  A call WITHOUT a bias
+// (every LLaMA layer: its projections have none) loses that wait, and where the launch is about one round of waves
+// it measured 10-27 % slower than the same call with a bias (2977 x 4096 fp16 with a residual: 18.6 against
+// 16.2 us; 2048 rows 12.7 against 11.2; fp32 1024-2304 rows alike).  kNormPacingLoad restores it: in place of the
+// absent bias vector the wave requests its gamma vector there and waits for it (the value is requested again
+// where it is used; both are cache hits).  With it the call without a bias takes what the call with one takes.
+// The launcher sets it for residual-without-bias launches that fit one round of waves and read more than 24 MiB;
+// below that size, over several rounds of waves, and for plain RMSNorm it measured 1-12 % slower and stays off.
+constexpr unsigned kNormPacingLoad = 0x40000000u;
+constexpr unsigned kNormInternalFlags = kNormStreamingOrder | kNormPacingLoad;
 
 // Which operands exist: known only at run time (the general kernel: uniform scalar branches), or fixed at
 // compile time for the kernels that launches of a few rows take (fused_norm_few_rows).
@@ -70,6 +81,7 @@ __device__ __forceinline__ void norm_rows_body(T* residual, T* out, const T* bia
     const bool has_bias = OPS == kOpsRuntime ? bias != nullptr : OPS == kOpsResidualBias;
     const bool literal_order = OPS == kOpsRuntime && (flags & ISP_NORM_RESIDUAL_EXCLUDES_BIAS) != 0;
     const bool streaming = OPS == kOpsRuntime && (flags & kNormStreamingOrder) != 0;
+    const bool pacing = OPS == kOpsRuntime && (flags & kNormPacingLoad) != 0;
     const size_t base = (size_t)(live ? row : 0) * (size_t)hidden;
     T* out_row = out + base;
     T* rsd_row = residual + base;  // dereferenced only when has_res
@@ -104,6 +116,11 @@ __device__ __forceinline__ void norm_rows_body(T* residual, T* out, const T* bia
             const int vi = lane + j * ROW_THREADS;
             vec16 vb;
             if (has_bias) vb = load16(bias + (size_t)vi * VEC);
+            else if (pacing) {
+                // no bias to wait for: wait for this vector's gamma instead (see kNormPacingLoad)
+                vb = load16(gamma + (size_t)vi * VEC);
+                asm volatile("" : "+v"(vb.w[0]) : : "memory");
+            }
             asm volatile("" ::: "memory");  // step 3: the next vector's bias is not requested early
             if (has_res) Elem<T>::sum(vo[j], vr[j], x[j]);
             else Elem<T>::unpack(vo[j], x[j]);
@@ -320,6 +337,7 @@ struct NormPlan {
     int wpr, nv, store, block_big;
     bool streaming;  // kNormStreamingOrder
     bool few;        // the launch occupies less than a quarter of the device: fused_norm_few_rows if it has the shape
+    bool pacing;     // kNormPacingLoad
 };
 
 template <typename T>
@@ -361,7 +379,7 @@ inline int few_rows_ops(bool has_res, bool has_bias, unsigned flags) {
 
 // The launch configuration for `tokens` rows of `nvec` 16-byte vectors.
 template <typename T>
-static NormPlan plan_norm(int tokens, int nvec, bool fused) {
+static NormPlan plan_norm(int tokens, int nvec, bool fused, bool has_bias = true) {
     auto vectors_per_lane = [nvec](int w) { return (nvec + kWave * w - 1) / (kWave * w); };
     // in place on both tensors: plain non-temporal stores measured best (write-through costs 2 %) -- except
     // where a launch writes no more than 1 MiB: ordinary stores, which the L2 acknowledges, then end the
@@ -417,7 +435,12 @@ static NormPlan plan_norm(int tokens, int nvec, bool fused) {
     const int order = tuning(ISP_TUNE_NORM_ORDER);
     const bool streaming = order == 2;
     const bool few = !streaming && order != 3 && (long long)tokens * wpr * 4 <= (long long)resident_waves();
-    return {wpr, vectors_per_lane(wpr), kind, big ? 1 : 0, streaming, few};
+    // see kNormPacingLoad; knob values 4 / 5 switch it off / on for every residual-without-bias launch
+    const bool one_round = (long long)tokens <= resident_rows(norm_variant<T>(wpr, vectors_per_lane(wpr), kind, big));
+    const size_t read_bytes = (size_t)tokens * (size_t)nvec * 16u * 2u;
+    const bool pacing = fused && !has_bias && !streaming && !few && order != 4 &&
+                        (order == 5 || (one_round && read_bytes > (24u << 20)));
+    return {wpr, vectors_per_lane(wpr), kind, big ? 1 : 0, streaming, few, pacing};
 }
 
 template <typename T>
@@ -438,9 +461,9 @@ static int fused_norm(void* residual_, void* out_, const void* bias_, const void
                         (hidden / VEC) <= kMaxNv * kWave * kMaxWpr;
     if (!vec_ok) {
         hipLaunchKernelGGL((fused_norm_generic<T>), dim3((unsigned)tokens), dim3(kBlock), 0, s,
-                           residual, out, bias, gamma, eps, tokens, hidden, flags & ~kNormStreamingOrder);
+                           residual, out, bias, gamma, eps, tokens, hidden, flags & ~kNormInternalFlags);
     } else {
-        const NormPlan plan = plan_norm<T>(tokens, hidden / VEC, residual != nullptr);
+        const NormPlan plan = plan_norm<T>(tokens, hidden / VEC, residual != nullptr, bias != nullptr);
         const int ops = few_rows_ops(residual != nullptr, bias != nullptr, flags);
         const NormFewKernel<T> few =
             plan.few && ops != kOpsRuntime ? norm_few_variant<T>(plan.wpr, plan.nv, plan.store, ops) : nullptr;
@@ -452,7 +475,8 @@ static int fused_norm(void* residual_, void* out_, const void* bias_, const void
             const NormVariant<T> v = norm_variant<T>(plan.wpr, plan.nv, plan.store, plan.block_big != 0);
             const dim3 grid((unsigned)((tokens + v.rows_per_block - 1) / v.rows_per_block));
             hipLaunchKernelGGL(v.kernel, grid, dim3(v.block), 0, s, residual, out, bias, gamma, eps, tokens, hidden,
-                               (flags & ~kNormStreamingOrder) | (plan.streaming ? kNormStreamingOrder : 0u));
+                               (flags & ~kNormInternalFlags) | (plan.streaming ? kNormStreamingOrder : 0u) |
+                                   (plan.pacing ? kNormPacingLoad : 0u));
         }
     }
     return note_launch(hipGetLastError());

@@ -62,7 +62,7 @@ def test_norm_every_vectors_per_lane_waves_per_row_store_kind_and_workgroup_size
         # the row sum is one fixed tree whatever the split of the row over waves and vectors per lane
         # order 1: the default (seven rows take the few-rows kernels where one exists), 2: streaming, 3: the general
         # kernel also for few rows
-        for split, store, block, order in itertools.product((1, 2, 4, 8, 16), (1, 2, 3), (256, 512), (1, 2, 3)):
+        for split, store, block, order in itertools.product((1, 2, 4, 8, 16), (1, 2, 3), (256, 512), (1, 2, 3)):  # noqa: E501
             say("norm %s hidden=%d waves/row=%d store=%d block=%d order=%d" % (dtype.__name__, hidden, split, store,
                                                                                  block, order))
             got = with_knobs({capi.TUNE_NORM_WAVES_PER_ROW: split, capi.TUNE_NORM_STORE: store,
@@ -125,6 +125,56 @@ def test_norm_few_rows_kernels_match_the_general_kernel_and_the_oracle(isp, orac
     assert lib.isp_norm_launch_variant(es, 4, vec * 64 * 16 * 4, 1, 0, 0) == 0
     assert lib.isp_norm_launch_variant(es, 16384, 4096, 1, 0, 0) == 0
     assert with_knobs({capi.TUNE_NORM_STORE: 3}, lambda: lib.isp_norm_launch_variant(es, 4, 4096, 1, 0, 0)) == 0
+
+
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+def test_norm_pacing_load_gives_the_same_bits(isp, oracle, dtype):
+    """A call with a residual and no bias may wait for a gamma vector where the bias vector would arrive (a matter
+    of timing only: knob order 5 forces it, 4 forbids it).  Same bits with and without, in every split of the row,
+    and the oracle's results at the size where the launcher switches it on by itself."""
+    from inferspore_amd import capi
+    vec = 8 if dtype == np.float16 else 4
+    for wpr, nv in ((1, 1), (2, 2), (4, 4), (8, 8), (16, 2)):
+        hidden = vec * 64 * wpr * nv - (vec if nv > 1 else 0)
+        tokens = 300   # beyond the few-rows kernels for every split
+        res, out, _, gamma = norm_inputs(tokens, hidden, dtype, seed=7 * wpr + nv)
+        d_gamma = dev(gamma)
+
+        def run():
+            d_res, d_out = dev(res), dev(out)
+            isp.fused_add_bias_residual_rmsnorm(d_res, d_out, None, d_gamma, 1e-5)
+            return d_res.cpu().numpy(), d_out.cpu().numpy()
+
+        e_res, e_out = oracle.fused_norm(res, out, None, gamma, 1e-5)
+        for block in (256, 512):
+            say("pacing load %s hidden=%d waves/row=%d block=%d" % (dtype.__name__, hidden, wpr, block))
+            base = with_knobs({capi.TUNE_NORM_WAVES_PER_ROW: wpr, capi.TUNE_NORM_BLOCK_THREADS: block,
+                               capi.TUNE_NORM_ORDER: 4}, run)
+            paced = with_knobs({capi.TUNE_NORM_WAVES_PER_ROW: wpr, capi.TUNE_NORM_BLOCK_THREADS: block,
+                                capi.TUNE_NORM_ORDER: 5}, run)
+            assert np.array_equal(base[0], e_res) and np.array_equal(paced[0], base[0])
+            assert np.array_equal(paced[1], base[1])
+            if dtype == np.float32:
+                assert_f32_close(base[1], e_out, "norm hidden %d" % hidden)
+            else:
+                assert_f16_close(base[1], e_out, "norm hidden %d" % hidden, max_mismatch_fraction=0.05)
+    # 2048 x 4096 with a residual and no bias: the size the default switches the wait on for
+    res, out, _, gamma = norm_inputs(2048, 4096, dtype, seed=99)
+    d_gamma = dev(gamma)
+
+    def big():
+        d_res, d_out = dev(res), dev(out)
+        isp.fused_add_bias_residual_rmsnorm(d_res, d_out, None, d_gamma, 1e-5)
+        return d_res.cpu().numpy(), d_out.cpu().numpy()
+
+    default = big()
+    off = with_knobs({capi.TUNE_NORM_ORDER: 4}, big)
+    e_res, e_out = oracle.fused_norm(res, out, None, gamma, 1e-5)
+    assert np.array_equal(default[0], e_res) and np.array_equal(default[0], off[0]) and np.array_equal(default[1], off[1])
+    if dtype == np.float32:
+        assert_f32_close(default[1], e_out, "norm 2048 x 4096 without bias")
+    else:
+        assert_f16_close(default[1], e_out, "norm 2048 x 4096 without bias", max_mismatch_fraction=0.05)
 
 
 @pytest.mark.parametrize("dtype", [np.float16, np.float32])
