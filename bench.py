@@ -386,6 +386,9 @@ def make_workloads(torch, lib, stream_handle, rotate):
     def copy(nbytes):
         return make_copy_workload(torch, lib, st, nbytes, rotate)
 
+    if rotate == "copy-curve":
+        return [("calibration_copy_%dMiB_traffic" % mib, (lambda mib=mib: copy((mib << 20) // 2)))
+                for mib in (1, 2, 4, 8, 16, 24, 32, 48, 64, 96, 128, 192, 256, 384, 512, 1024)]
     if rotate == "gather-locality":
         return [("embedding_f16_8192x4096_v32000" + ("_runs_of_%d" % n if n != 1 else ""),
                  (lambda n=n: embedding(id_run=n))) for n in (1, 2, 4, 8, 32, 0)] + [("calibration_copy_128MiB_traffic", lambda: copy(64 << 20))]
@@ -1002,32 +1005,36 @@ def main():
     gate = QueueGate(torch, lib, stream)
     dispatch_log.append(["gate_calibration", "isp::copy_vec<1>", QueueGate.CALIBRATION_LAUNCHES])
 
+    def side_study(line, results):
+        """The special modes print the same per-workload records and launch log as --kernels-only, so that
+        `python -m inferspore_amd.profile_summary` can summarise a rocprofv3 trace of them too."""
+        line.update({"steps": a.steps, "warmup": a.warmup, "lead_in": LEAD_IN, "dispatch_log": dispatch_log,
+                     "regions_ahead": {r["workload"]: r["regions_ahead"] for r in results},
+                     "roofline": {"per_config": {r["workload"]: compact(r) for r in results}}})
+        print(json.dumps(line))
+
     if a.copy_curve:
-        points = []
-        for mib in (8, 16, 24, 32, 48, 64, 96, 128, 192, 256, 384, 512, 1024):
-            with torch.cuda.stream(stream):
-                w = make_copy_workload(torch, lib, handle, (mib << 20) // 2)
-            torch.cuda.synchronize()
-            r = measure(torch, w, a.steps, a.warmup, regions, stream, traffic, gate)
-            points.append({"traffic_MiB": mib, "us_per_launch": r["ms_per_launch_events"] * 1e3, "GBps": r["GBps"],
-                           "frac_of_hbm_peak": r["frac_of_hbm_peak"]})
-            del w
-        # least-squares line  time = fixed + bytes / rate  over the points
-        xs = [p["traffic_MiB"] * 2.0 ** 20 for p in points]
-        ys = [p["us_per_launch"] for p in points]
+        results = run_all("copy-curve")
+        points = [{"traffic_MiB": r["algorithmic_bytes"] >> 20, "us_per_launch": r["ms_per_launch_events"] * 1e3,
+                   "GBps": r["GBps"], "frac_of_hbm_peak": r["frac_of_hbm_peak"]} for r in results]
+        # least-squares line  time = fixed + bytes / rate  over the points from 16 MiB up
+        fit = [p for p in points if p["traffic_MiB"] >= 16]
+        xs = [p["traffic_MiB"] * 2.0 ** 20 for p in fit]
+        ys = [p["us_per_launch"] for p in fit]
         n = len(xs)
         mx, my = sum(xs) / n, sum(ys) / n
         slope = sum((x - mx) * (y - my) for x, y in zip(xs, ys)) / sum((x - mx) ** 2 for x in xs)
-        print(json.dumps({"metric": "plain copy (isp_calibration_copy) vs traffic per launch", "unit": "GB/s",
-                          "points": points, "fit": {"fixed_us": my - slope * mx, "asymptotic_GBps": 1e-3 / slope}}))
+        side_study({"metric": "plain copy (isp_calibration_copy) vs traffic per launch", "unit": "GB/s", "points": points,
+                    "fit": {"fixed_us": my - slope * mx, "asymptotic_GBps": 1e-3 / slope, "over": "16 MiB .. 1 GiB"}},
+                   results)
         return
 
     if a.gather_locality:
-        pts = run_all("gather-locality")
-        print(json.dumps({"metric": "embedding gather vs locality of the token ids (8192 ids, 32000 x 4096 fp16 table)",
-                          "unit": "us per launch",
-                          "points": {r["workload"]: {"us": round(r["ms_per_launch_events"] * 1e3, 3),
-                                                     "GBps": round(r["GBps"], 1)} for r in pts}}))
+        results = run_all("gather-locality")
+        side_study({"metric": "embedding gather vs locality of the token ids (8192 ids, 32000 x 4096 fp16 table)",
+                    "unit": "us per launch",
+                    "points": {r["workload"]: {"us": round(r["ms_per_launch_events"] * 1e3, 3),
+                                               "GBps": round(r["GBps"], 1)} for r in results}}, results)
         return
 
     results = run_all(True)

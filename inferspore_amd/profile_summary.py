@@ -88,13 +88,76 @@ def tail_of(values, skip):
     return values[skip:] if len(values) > skip else values
 
 
+def summarise_layer(a):
+    """Per-layer kernel breakdown of a traced build/bin/bench_context_layer run: RUN/layer/layer.json is the program's
+    stdout, the trace CSV lies below RUN/layer.  The layer's kernels repeat with a fixed period; the timed iterations
+    are the last `iterations` periods of the trace."""
+    import re
+    ldir = os.path.join(a.run, "layer")
+    with open(os.path.join(ldir, "layer.json")) as f:
+        text = f.read()
+    rec = json.loads([l for l in text.splitlines() if l.startswith("{")][-1])
+    cmd = [l for l in text.splitlines() if l.startswith("command: ")]
+    with open(find_one(ldir, "*kernel_trace.csv"), newline="") as f:
+        rows = list(csv.DictReader(f))
+    rows.sort(key=lambda r: int(r["Start_Timestamp"]))
+
+    def short(n):
+        if n.startswith("Cijk_"):
+            return "hipBLASLt GEMM kernels (Cijk_*)"
+        m = re.search(r"context_attention_f16ILi(\d+)E", n)   # a name the profiler leaves mangled
+        if m:
+            return "isp_layers::context_attention_f16<%s> (fused attention)" % m.group(1)
+        return re.sub(r"^void ", "", n).split("(")[0]
+
+    names = [short(r["Kernel_Name"]) for r in rows]
+    iters = int(rec["iterations"])
+    per = next(p for p in range(2, 64) if len(names) >= 3 * p and names[-p:] == names[-2 * p:-p] == names[-3 * p:-2 * p])
+    tail = rows[-iters * per:]
+    agg = {}
+    for r in tail:
+        k = agg.setdefault(short(r["Kernel_Name"]), [0, 0])
+        k[0] += 1
+        k[1] += int(r["End_Timestamp"]) - int(r["Start_Timestamp"])
+    total = sum(v[1] for v in agg.values())
+    span = sum(int(tail[i * per + per - 1]["End_Timestamp"]) - int(tail[i * per]["Start_Timestamp"]) for i in range(iters))
+    out = ["rocprofv3 kernel-trace summary: the C++ context-decoder layer (LlamaContextDecoderLayer<half>) at LLaMA-2-7B shape,",
+           "batch %d, max_q_len %d, %d valid tokens, %s attention" % (rec["batch"], rec["max_q_len"], rec["valid_tokens"], rec["attention"]), "",
+           "command (run from /tmp with TMPDIR=/tmp on the MI355X box; the binary is built by `python -m inferspore_amd.build`):",
+           "  " + (cmd[-1][len("command: "):] if cmd else "rocprofv3 --kernel-trace --stats --output-format csv -d RUN/layer -o layer -- build/bin/bench_context_layer ..."),
+           "  python3 -m inferspore_amd.profile_summary RUN --layer --out profiles", "",
+           "per layer over the %d timed iterations (%d kernels per layer; warm-up iterations, which include the one-off" % (iters, per),
+           "algorithm-selection runs of the GEMM plan cache, are left out); the program's own figure for the same run: %.3f ms per layer" % rec["ms_per_layer"]]
+    for k, v in sorted(agg.items(), key=lambda kv: -kv[1][1]):
+        out.append("%-62s %4.1f calls/layer %8.1f us/layer %5.1f%%" % (k, v[0] / iters, v[1] / iters / 1e3, 100.0 * v[1] / total))
+    out.append("sum of kernel time per layer: %.1f us; first kernel start to last kernel end per layer: %.1f us"
+               % (total / iters / 1e3, span / iters / 1e3))
+    out += ["", "one layer's kernels in call order (last iteration, us):"]
+    for r in tail[-per:]:
+        out.append("  %-62s %8.2f" % (short(r["Kernel_Name"]), (int(r["End_Timestamp"]) - int(r["Start_Timestamp"])) / 1e3))
+    name = "context_decoder_layer_cpp_llama2_7b_b%d_s%d%s.kernel_trace_stats.txt" % (
+        rec["batch"], rec["max_q_len"], "" if rec["attention"] == "fused" else "_" + rec["attention"])
+    with open(os.path.join(a.out, name), "w") as f:
+        f.write("\n".join(out) + "\n")
+    print("profile_summary: wrote %s" % os.path.join(a.out, name))
+    return 0
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("run", help="directory with trace/ and one sub-directory per counter run")
     ap.add_argument("--out", default="profiles")
+    ap.add_argument("--prefix", default="all_kernels_benchmark_shapes", help="file name stem of the summaries")
+    ap.add_argument("--title", default="every kernel of the library at its benchmark shape (bench.py, all workloads)")
+    ap.add_argument("--bench-args", default="--kernels-only", help="the arguments bench.py was run with")
+    ap.add_argument("--layer", action="store_true",
+                    help="RUN/layer holds a kernel trace of build/bin/bench_context_layer and its stdout (layer.json): "
+                         "write the per-layer kernel breakdown instead")
     a = ap.parse_args()
     os.makedirs(a.out, exist_ok=True)
-    prefix = os.path.join(a.out, "all_kernels_benchmark_shapes")
+    if a.layer:
+        return summarise_layer(a)
+    prefix = os.path.join(a.out, a.prefix)
 
     # ---------------------------------------------------------------- kernel trace
     tdir = os.path.join(a.run, "trace")
@@ -126,10 +189,11 @@ def main():
                 sel += v[(warm + r * steps) * per_step:(warm + (r + 1) * steps) * per_step]
         return sel
 
-    out = ["rocprofv3 kernel-trace summary: every kernel of the library at its benchmark shape (bench.py, all workloads)", "",
+    extra = "" if a.prefix == "all_kernels_benchmark_shapes" else " --prefix %s --bench-args '%s' --title '...'" % (a.prefix, a.bench_args)
+    out = ["rocprofv3 kernel-trace summary: " + a.title, "",
            "command (run from /tmp with TMPDIR=/tmp on the MI355X box):",
-           "  rocprofv3 --kernel-trace --stats --output-format csv -d RUN/trace -o bench -- python3 bench.py --kernels-only",
-           "  python3 -m inferspore_amd.profile_summary RUN --out profiles",
+           "  rocprofv3 --kernel-trace --stats --output-format csv -d RUN/trace -o bench -- python3 bench.py " + a.bench_args,
+           "  python3 -m inferspore_amd.profile_summary RUN --out profiles" + extra,
            "  (--steps %d --warmup %d; launches rotate over >1 GiB of buffer sets; warm-up, gate and lead-in dispatches excluded)"
            % (steps, bench["warmup"]), "",
            "per workload from the kernel trace -- durations in microseconds; GB/s = algorithmic bytes / average duration.",
@@ -166,6 +230,17 @@ def main():
             if "isp::" in r["Name"]:
                 out.append("  %s, %s, %.0f, %s, %s" % (r["Name"].split("(")[0].replace("void ", ""), r["Calls"],
                                                        float(r["AverageNs"]), r["MinNs"], r["MaxNs"]))
+    plain = os.path.join(a.run, "plain.json")
+    if os.path.exists(plain):
+        with open(plain) as f:
+            pj = json.loads([l for l in f.read().splitlines() if l.startswith("{")][-1])
+        out += ["", "the same command without the profiler (python3 bench.py %s): HIP-event time per launch" % a.bench_args,
+                "%-48s %10s %8s %8s" % ("workload", "us", "GB/s", "of 8TB/s")]
+        for w, rec in pj["roofline"]["per_config"].items():
+            out.append("%-48s %10.2f %8.0f %7.1f%%" % (w, rec["us"], rec["GBps"], 100.0 * rec["frac"]))
+        if "fit" in pj:
+            out.append("least-squares line over %s: time = %.2f us + bytes / %.0f GB/s"
+                       % (pj["fit"].get("over", "the points"), pj["fit"]["fixed_us"], pj["fit"]["asymptotic_GBps"]))
     with open(prefix + ".kernel_trace_stats.txt", "w") as f:
         f.write("\n".join(out) + "\n")
 
