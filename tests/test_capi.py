@@ -78,6 +78,29 @@ def test_argument_validation_returns_before_any_launch(lib):
     assert call(hs=1024, rot=1024) == capi.ERR_UNSUPPORTED
 
 
+def test_norm_launch_queries_need_no_device(lib):
+    """isp_norm_launch_config / isp_norm_launch_variant only describe what a call would launch: they work without
+    a GPU (device facts fall back to the MI355X's) and reject what the norm entry points reject."""
+    from inferspore_amd import capi
+    out = [ctypes.c_int() for _ in range(4)]
+    refs = [ctypes.byref(x) for x in out]
+    assert lib.isp_norm_launch_config(2, 2048, 4096, 1, *refs) == capi.OK
+    assert out[0].value in (1, 2, 4, 8, 16) and out[1].value in (1, 2, 4, 8) and out[2].value in (256, 512, 1024)
+    assert lib.isp_norm_launch_config(2, 0, 4096, 1, *refs) == capi.ERR_BAD_SHAPE
+    assert lib.isp_norm_launch_config(3, 8, 4096, 1, *refs) == capi.ERR_BAD_SHAPE          # no such element size
+    assert lib.isp_norm_launch_config(2, 8, 4095, 1, *refs) == capi.ERR_UNSUPPORTED        # not whole vectors: scalar kernel
+    # a decode-step norm takes the few-rows kernel, a prefill-sized one the general kernel; the reference's literal
+    # residual order and a bias without a residual are outside the few-rows kernels
+    assert lib.isp_norm_launch_variant(2, 16, 4096, 1, 0, 0) == 1
+    assert lib.isp_norm_launch_variant(4, 64, 4096, 0, 0, 0) == 1
+    assert lib.isp_norm_launch_variant(2, 4096, 4096, 1, 0, 0) == 0
+    assert lib.isp_norm_launch_variant(2, 16, 4096, 1, 1, capi.NORM_RESIDUAL_EXCLUDES_BIAS) == 0
+    assert lib.isp_norm_launch_variant(2, 16, 4096, 0, 1, 0) == 0
+    assert lib.isp_norm_launch_variant(2, -1, 4096, 1, 0, 0) == capi.ERR_BAD_SHAPE
+    assert lib.isp_norm_launch_variant(8, 16, 4096, 1, 0, 0) == capi.ERR_BAD_SHAPE
+    assert lib.isp_norm_launch_variant(4, 16, 4098, 1, 0, 0) == capi.ERR_UNSUPPORTED
+
+
 def test_python_layer_refuses_cpu_tensors():
     import torch
     from inferspore_amd import ops
