@@ -239,8 +239,10 @@ def make_workloads(torch, lib, stream_handle, rotate):
         batch, seq, tokens, lens_d, po = padded_batch()
         w.name, w.dtype, w.tokens = "qkv_bias_rope_transpose_%s_b8_s512%s" % (sfx, tag), sfx, tokens
         flag = "true" if with_bias else "false"
-        if es == 2 and hs == 128 and hn % 32 == 0 and kvn % 32 == 0:
-            w.kernel = "isp::qkv_rope_lean_f16<2, %s, false>" % flag
+        if es == 2 and hs == 128 and hn % 4 == 0 and kvn % 4 == 0:
+            w.kernel = "isp::qkv_rope_lean_f16<2, %s, false, %s>" % (flag, "false" if hn % 32 == 0 and kvn % 32 == 0 else "true")
+        elif es == 4 and hs == 128 and hn % 2 == 0 and kvn % 2 == 0:
+            w.kernel = "isp::qkv_rope_lean_f32<2, %s, false, %s>" % (flag, "false" if hn % 16 == 0 and kvn % 16 == 0 else "true")
         else:
             w.kernel = "isp::qkv_rope_wave<%s, %d, 2, 4, %s>" % ("__half" if es == 2 else "float", hs, flag)
         w.bytes_per_launch = tokens * (2 * (hn + 2 * kvn) * hs * es + 4) + 2 * batch * 4
@@ -283,14 +285,14 @@ def make_workloads(torch, lib, stream_handle, rotate):
         caches = [[torch.zeros((1, batch, kvn, max_seq, hs), device=dev, dtype=tdtype) for _ in range(2)] for _ in range(R)]
         w.keep = (lens_d, po, hist, bias, ins, qs, caches)
         if fused:
-            w.name, w.kernel = "qkv_bias_rope_transpose_append_f16_b8_s512_S1024", "isp::qkv_rope_lean_f16<2, true, true>"
+            w.name, w.kernel = "qkv_bias_rope_transpose_append_f16_b8_s512_S1024", "isp::qkv_rope_lean_f16<2, true, true, false>"
             w.bind(lib.isp_qkv_bias_rope_transpose_append_f16,
                    [(qs[j].data_ptr(), None, None, caches[j][0].data_ptr(), caches[j][1].data_ptr(), 0, max_seq,
                      ins[j].data_ptr(), bias.data_ptr(), po.data_ptr(), hist.data_ptr(), lens_d.data_ptr(), batch, seq,
                      tokens, hn, kvn, hs, hs, 10000.0, st) for j in range(R)])
         else:
             w.name = "qkv_bias_rope_transpose_then_concat_kv_f16_b8_s512_S1024"
-            w.kernel = "isp::qkv_rope_lean_f16<2, true, false> + isp::concat_kv_vec<256>"
+            w.kernel = "isp::qkv_rope_lean_f16<2, true, false, false> + isp::concat_kv_vec<256>"
             kvs = [[torch.zeros((batch, kvn, seq, hs), device=dev, dtype=tdtype) for _ in range(2)] for _ in range(R)]
             w.keep += (kvs,)
             w.bind_pair(lib.isp_qkv_bias_rope_transpose_f16,
@@ -423,6 +425,7 @@ def make_workloads(torch, lib, stream_handle, rotate):
          lambda: norm("fused_add_bias_residual_rmsnorm_f32_2048x4096", 2048, 4096, torch.float32, True)),
         ("embedding_f32_8192x4096_v32000", lambda: embedding(torch.float32)),
         ("qkv_bias_rope_transpose_f32_b8_s512", lambda: qkv(torch.float32)),
+        ("qkv_bias_rope_transpose_f32_b8_s512_no_bias", lambda: qkv(torch.float32, tag="_no_bias", with_bias=False)),
         ("swiglu_f32_prefill_8192x11008", lambda: swiglu(8192, "prefill", torch.float32)),
         ("calibration_copy_2MiB_traffic", lambda: copy(1 << 20)),
         ("calibration_copy_16MiB_traffic", lambda: copy(8 << 20)),

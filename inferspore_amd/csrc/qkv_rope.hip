@@ -18,11 +18,12 @@
 //     while their own loads are in flight (the reference evaluates powf + cos + sin for every
 //     (head, d): 48 to 96 times more transcendental work);
 //   * the streamed loads are issued before anything that depends on padding_offset / history;
-//   * two kernels share this: qkv_rope_lean_f16 for the common LLaMA shape (one 16-byte vector per
-//     lane, partner exchange by DPP, scalar address arithmetic) and qkv_rope_wave for every other
-//     vectorisable shape and for fp32 (a lane owns 16 bytes at d = VEC*g and the 16 bytes of its
-//     rotation partners at d + hs/2, so the rotate-half pairing needs no cross-lane exchange); both
-//     read and write whole 128-byte lines of the 256-byte head rows and give identical bits;
+//   * the kernels that share this: qkv_rope_lean_f16 / qkv_rope_lean_f32 for the common LLaMA shape
+//     (one 16-byte vector per lane, the rotation partner fetched from another lane in the VALU, scalar
+//     address arithmetic), qkv_rope_lean64_f16 for 64-element heads, and qkv_rope_wave for every other
+//     vectorisable shape (a lane owns 16 bytes at d = VEC*g and the 16 bytes of its rotation partners
+//     at d + hs/2, so the rotate-half pairing needs no cross-lane exchange); all read and write whole
+//     128-byte lines of the head rows and give identical bits;
 //   * stores are non-temporal write-through (q, k, v are consumed by a later kernel).
 #include <math.h>
 #include <stddef.h>
@@ -326,11 +327,11 @@ __global__ __launch_bounds__(kWave * WAVES) void qkv_rope_rows64_f16(
     if (cache) store16_sel<ST>(cache + col, out);
 }
 
-// The common LLaMA shape (fp16, head size 128 fully rotated, q and kv head counts multiples of 32)
+// The common LLaMA shape (fp16, head size 128 fully rotated, q and kv head counts multiples of 4)
 // with as few instructions per wave as the arithmetic allows, because at one 16-byte vector per
 // lane a wave moves only 1 KiB and anything above ~100 vector instructions per wave shows up in
-// the run time.  One vector per lane: 512 threads carry the 32 heads of one group (all q, all k or
-// all v) of one token, every load and store instruction of a wave covers 4 whole head rows.  The
+// the run time.  One vector per lane: 512 threads carry a group of 32 heads of one token (all q, all
+// k or all v, unless SPLIT), every load and store instruction of a wave covers 4 whole head rows.  The
 // rotation partner (d +- 64) is 8 lanes away and comes through a DPP row rotation; (cos, sin) are
 // evaluated once per workgroup by its first wave and stored twice, as (c, -s) for the lower and
 // (c, s) for the upper half of a row, so that both halves run out = c * x + t * partner; row,
@@ -338,29 +339,42 @@ __global__ __launch_bounds__(kWave * WAVES) void qkv_rope_rows64_f16(
 // rotate_pair(), so the results are bit-identical to the other kernels of this file.  BIAS is a
 // template argument so that each variant has a fixed sequence of loads and the compiler's waits
 // are exact for it; so is APPEND (k and v rows also, or only, into the KV cache).
+// SPLIT = false: head counts in multiples of 32, so a workgroup's 32 heads belong to one plane and all
+// placement arithmetic is workgroup-uniform.  SPLIT = true: head counts in multiples of 4 (grouped-query
+// shapes, 40-head models): each wave places its own 4 heads, the q / k / v boundaries and the end of the
+// token's heads may fall between the waves of a workgroup, and a wave without heads reads rows that exist,
+// stays until the barrier and leaves.
 // `tab` MUST stay the first parameter: first_argument_word() reads it at byte 0 of the argument
 // block (the launcher asserts its offset, and a test checks every coefficient through the ABI).
-template <int ST, bool BIAS, bool APPEND>
+template <int ST, bool BIAS, bool APPEND, bool SPLIT>
 __global__ __launch_bounds__(512) void qkv_rope_lean_f16(
     RopeDivisors tab, __half* q, __half* k, __half* v, const __half* qkv, const __half* bias,
     const int32_t* __restrict__ padding_offset, const int32_t* __restrict__ history_length,
     unsigned positions, FastDiv seq, unsigned head_num, unsigned kv_head_num,
     KvAppend<__half> ap) {
-    constexpr unsigned ROW_BYTES = 256, GROUP = 32;
+    constexpr unsigned ROW_BYTES = 256, GROUP = 32, WAVE_HEADS = 4;
     const unsigned tid = threadIdx.x;
     const unsigned token = blockIdx.x;
-    const unsigned first = blockIdx.y * GROUP;  // first head of this workgroup's group
+    // first head of this workgroup's group: 32 heads, or with SPLIT as many as the launch gave it waves for
+    const unsigned group_first = blockIdx.y * (SPLIT ? blockDim.x / (64u / WAVE_HEADS) : GROUP);
     const unsigned qkv_heads = head_num + 2 * kv_head_num;
+    // the heads this wave (SPLIT) or this workgroup places start at `first`; `slot` = the lane's 16-byte
+    // slot counted from there
+    const unsigned first =
+        SPLIT ? group_first + (unsigned)__builtin_amdgcn_readfirstlane(tid >> 6) * WAVE_HEADS : group_first;
+    const unsigned slot = SPLIT ? (tid & 63u) : tid;
+    const bool live = !SPLIT || first < qkv_heads;  // wave-uniform
+    const unsigned first_read = live ? first : 0u;
 
     // loads in the order divisor, streamed row, bias, and kept in it (see first_argument_word)
     const float my_divisor = first_argument_word(tid & 63u);
     (void)tab;
     asm volatile("" ::: "memory");
-    const char* src = reinterpret_cast<const char*>(qkv) + ((size_t)token * qkv_heads + first) * ROW_BYTES;
-    const vec16 raw = load16_stream(src + tid * 16u);
+    const char* src = reinterpret_cast<const char*>(qkv) + ((size_t)token * qkv_heads + first_read) * ROW_BYTES;
+    const vec16 raw = load16_stream(src + slot * 16u);
     asm volatile("" ::: "memory");
     vec16 braw;
-    if (BIAS) braw = load16(reinterpret_cast<const char*>(bias) + (size_t)first * ROW_BYTES + tid * 16u);
+    if (BIAS) braw = load16(reinterpret_cast<const char*>(bias) + (size_t)first_read * ROW_BYTES + slot * 16u);
     asm volatile("" ::: "memory");  // keeps the loads in front of the lookups below
 
     const long long p = (long long)token + (long long)read_only_i32(padding_offset, (int)token);
@@ -379,31 +393,32 @@ __global__ __launch_bounds__(512) void qkv_rope_lean_f16(
         plane = v, plane_heads = kv_head_num, h0 = first - head_num - kv_head_num;
     }
     char* dst = reinterpret_cast<char*>(plane) + (((size_t)b * plane_heads + h0) * seq.d + s) * ROW_BYTES;
-    const unsigned lane_offset = (tid >> 4) * (seq.d * ROW_BYTES) + (tid & 15u) * 16u;  // head row, column
-    // the same group of rows in the KV cache (k and v groups only); all of it wave-uniform
+    const unsigned lane_offset = (slot >> 4) * (seq.d * ROW_BYTES) + (slot & 15u) * 16u;  // head row, column
+    // the same rows in the KV cache (k and v heads only); all of it wave-uniform
     char* cdst = nullptr;
     unsigned cache_lane_offset = 0;
+    bool idle = !live;  // nothing (more) to write for these heads
     if (APPEND && first >= head_num) {
         const long long row = append_row(ap, history_length, (int)b, (int)s);
         if (row >= 0) {
             cdst = reinterpret_cast<char*>(rotates ? ap.k_cache : ap.v_cache) +
                    (((size_t)b * plane_heads + h0) * (size_t)ap.max_seq_len + (size_t)row) * ROW_BYTES;
-            cache_lane_offset = (tid >> 4) * ((unsigned)ap.max_seq_len * ROW_BYTES) + (tid & 15u) * 16u;
+            cache_lane_offset = (slot >> 4) * ((unsigned)ap.max_seq_len * ROW_BYTES) + (slot & 15u) * 16u;
         }
-        if (plane == nullptr && cdst == nullptr) return;  // nothing to write for this group
+        if (plane == nullptr && cdst == nullptr) idle = true;
     }
-
-    if (!rotates && !BIAS) {  // v heads without bias: a plain move
+    if (!idle && !rotates && !BIAS) {  // v heads without bias: a plain move
         if (!APPEND || plane != nullptr) store16_sel<ST>(dst + lane_offset, raw);
         if (APPEND && cdst != nullptr) store16_sel<ST>(cdst + cache_lane_offset, raw);
-        return;
+        idle = true;
     }
+    if (!SPLIT && idle) return;  // workgroup-uniform without SPLIT; with it every wave goes on to the barrier
     // the coefficient table first: the first wave evaluates it while every wave's loads are in flight
     // Table layout [j][class][2]: class = tid & 15 names a lane's column and half row (16 classes),
     // j = 0..3 its four 16-byte reads of two (c, t) pairs each; the 16 classes of one j are
     // contiguous (256 bytes = all 64 banks), so the reads of a wave are conflict-free.
     __shared__ float2 cs[4][16][2];
-    if (rotates) {
+    if (SPLIT ? group_first < head_num + kv_head_num : rotates) {  // workgroup-uniform: its first wave rotates
         if (tid < 64) {
             const float2 coef = rope_coefficients(read_only_i32(history_length, (int)b) + (int)s, my_divisor);
             const unsigned g = tid >> 3, e = tid & 7u;  // pair tid = element e of column group g
@@ -412,6 +427,7 @@ __global__ __launch_bounds__(512) void qkv_rope_lean_f16(
         }
         __syncthreads();
     }
+    if (SPLIT && idle) return;
     float x[8], y[8];
     Elem<__half>::unpack(raw, x);
     if (BIAS) {
@@ -433,6 +449,120 @@ __global__ __launch_bounds__(512) void qkv_rope_lean_f16(
         for (int e = 0; e < 8; e++) y[e] = x[e];
     }
     const vec16 packed = Elem<__half>::pack(y);
+    if (!APPEND || plane != nullptr) store16_sel<ST>(dst + lane_offset, packed);
+    if (APPEND && cdst != nullptr) store16_sel<ST>(cdst + cache_lane_offset, packed);
+}
+
+// The same design for fp32 rows (head size 128 fully rotated, q and kv head counts multiples of 16, or of 2
+// with SPLIT): a head row is 512 bytes = 32 lanes of one 16-byte vector, a wave carries two rows and 512
+// threads the 16 heads of one group.  The rotation partner (d +- 64) is 16 lanes away, in the neighbouring row of 16 lanes:
+// v_permlane16_swap exchanges the odd rows of one register with the even rows of another, so applied to
+// two copies of x it leaves every lane with the value of its even-row neighbour in one result and of its
+// odd-row neighbour in the other, and a lane picks the one that is not its own.  Same operations per
+// element as rotate_pair(): bit-identical to qkv_rope_wave<float, ...>, which this replaces for that shape
+// (two vectors per lane there).
+// `tab` MUST stay the first parameter (first_argument_word).
+template <int ST, bool BIAS, bool APPEND, bool SPLIT>
+__global__ __launch_bounds__(512) void qkv_rope_lean_f32(
+    RopeDivisors tab, float* q, float* k, float* v, const float* qkv, const float* bias,
+    const int32_t* __restrict__ padding_offset, const int32_t* __restrict__ history_length,
+    unsigned positions, FastDiv seq, unsigned head_num, unsigned kv_head_num, KvAppend<float> ap) {
+    constexpr unsigned ROW_BYTES = 512, GROUP = 16, WAVE_HEADS = 2;
+    const unsigned tid = threadIdx.x;
+    const unsigned token = blockIdx.x;
+    const unsigned group_first = blockIdx.y * (SPLIT ? blockDim.x / (64u / WAVE_HEADS) : GROUP);
+    const unsigned qkv_heads = head_num + 2 * kv_head_num;
+    // SPLIT (head counts in multiples of 2 instead of 16): every wave places its own two heads
+    const unsigned first =
+        SPLIT ? group_first + (unsigned)__builtin_amdgcn_readfirstlane(tid >> 6) * WAVE_HEADS : group_first;
+    const unsigned slot = SPLIT ? (tid & 63u) : tid;
+    const bool live = !SPLIT || first < qkv_heads;  // wave-uniform
+    const unsigned first_read = live ? first : 0u;
+
+    const float my_divisor = first_argument_word(tid & 63u);
+    (void)tab;
+    asm volatile("" ::: "memory");
+    const char* src = reinterpret_cast<const char*>(qkv) + ((size_t)token * qkv_heads + first_read) * ROW_BYTES;
+    const vec16 raw = load16_stream(src + slot * 16u);
+    asm volatile("" ::: "memory");
+    vec16 braw;
+    if (BIAS) braw = load16(reinterpret_cast<const char*>(bias) + (size_t)first_read * ROW_BYTES + slot * 16u);
+    asm volatile("" ::: "memory");
+
+    const long long p = (long long)token + (long long)read_only_i32(padding_offset, (int)token);
+    if (p < 0 || p >= (long long)positions) return;  // workgroup-uniform
+    unsigned b, s;
+    seq.divmod((unsigned)p, b, s);
+
+    float* plane;
+    unsigned plane_heads, h0;
+    const bool rotates = first < head_num + kv_head_num;
+    if (first < head_num) {
+        plane = q, plane_heads = head_num, h0 = first;
+    } else if (rotates) {
+        plane = k, plane_heads = kv_head_num, h0 = first - head_num;
+    } else {
+        plane = v, plane_heads = kv_head_num, h0 = first - head_num - kv_head_num;
+    }
+    char* dst = reinterpret_cast<char*>(plane) + (((size_t)b * plane_heads + h0) * seq.d + s) * ROW_BYTES;
+    const unsigned lane_offset = (slot >> 5) * (seq.d * ROW_BYTES) + (slot & 31u) * 16u;  // head row, column
+    char* cdst = nullptr;
+    unsigned cache_lane_offset = 0;
+    bool idle = !live;  // nothing (more) to write for these heads
+    if (APPEND && first >= head_num) {
+        const long long row = append_row(ap, history_length, (int)b, (int)s);
+        if (row >= 0) {
+            cdst = reinterpret_cast<char*>(rotates ? ap.k_cache : ap.v_cache) +
+                   (((size_t)b * plane_heads + h0) * (size_t)ap.max_seq_len + (size_t)row) * ROW_BYTES;
+            cache_lane_offset = (slot >> 5) * ((unsigned)ap.max_seq_len * ROW_BYTES) + (slot & 31u) * 16u;
+        }
+        if (plane == nullptr && cdst == nullptr) idle = true;
+    }
+    if (!idle && !rotates && !BIAS) {  // v heads without bias: a plain move
+        if (!APPEND || plane != nullptr) store16_sel<ST>(dst + lane_offset, raw);
+        if (APPEND && cdst != nullptr) store16_sel<ST>(cdst + cache_lane_offset, raw);
+        idle = true;
+    }
+    if (!SPLIT && idle) return;  // workgroup-uniform without SPLIT; with it every wave goes on to the barrier
+    // Table layout [j][class][2]: class = tid & 31 names a lane's column and half row (16 classes of the
+    // lower half row with (c, -s), 16 of the upper with (c, s)), j = 0..1 its two 16-byte reads of two
+    // (c, t) pairs each; the 32 classes of one j are contiguous
+    __shared__ float2 cs[2][32][2];
+    if (SPLIT ? group_first < head_num + kv_head_num : rotates) {  // workgroup-uniform: its first wave rotates
+        if (tid < 64) {
+            const float2 coef = rope_coefficients(read_only_i32(history_length, (int)b) + (int)s, my_divisor);
+            const unsigned g = tid >> 2, e = tid & 3u;  // pair tid = element e of column group g
+            cs[e >> 1][g][e & 1u] = make_float2(coef.x, -coef.y);
+            cs[e >> 1][g + 16][e & 1u] = coef;
+        }
+        __syncthreads();
+    }
+    if (SPLIT && idle) return;
+    float x[4], y[4];
+    Elem<float>::unpack(raw, x);
+    if (BIAS) {
+        float bv[4];
+        Elem<float>::unpack(braw, bv);
+#pragma unroll
+        for (int e = 0; e < 4; e++) x[e] += bv[e];
+    }
+    if (rotates) {
+        const unsigned cls = tid & 31u;
+        const bool upper = (tid & 16u) != 0;  // odd row of 16 lanes: holds x[d + 64], its partner sits one row down
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            const float2 t = cs[e >> 1][cls][e & 1];
+            const unsigned bits = __float_as_uint(x[e]);
+            const auto r = __builtin_amdgcn_permlane16_swap(bits, bits, false, false);
+            // r[0]: every row pair holds its even row's values, r[1]: its odd row's
+            const float other = __uint_as_float(upper ? r[0] : r[1]);
+            y[e] = __fmaf_rn(t.x, x[e], t.y * other);
+        }
+    } else {
+#pragma unroll
+        for (int e = 0; e < 4; e++) y[e] = x[e];
+    }
+    const vec16 packed = Elem<float>::pack(y);
     if (!APPEND || plane != nullptr) store16_sel<ST>(dst + lane_offset, packed);
     if (APPEND && cdst != nullptr) store16_sel<ST>(cdst + cache_lane_offset, packed);
 }
@@ -572,13 +702,16 @@ template <typename A0, typename... A>
 struct FirstParameter<void (*)(A0, A...)> {
     using type = A0;
 };
-static_assert(std::is_same<FirstParameter<decltype(&qkv_rope_lean_f16<kStorePlain, false, false>)>::type,
+static_assert(std::is_same<FirstParameter<decltype(&qkv_rope_lean_f16<kStorePlain, false, false, false>)>::type,
                            RopeDivisors>::value &&
                   offsetof(RopeDivisors, div) == 0,
               "qkv_rope_lean_f16 must take the divisor table as its first parameter");
 static_assert(std::is_same<FirstParameter<decltype(&qkv_rope_lean64_f16<kStorePlain, false, false>)>::type,
                            RopeDivisors>::value,
               "qkv_rope_lean64_f16 must take the divisor table as its first parameter");
+static_assert(std::is_same<FirstParameter<decltype(&qkv_rope_lean_f32<kStorePlain, false, false, false>)>::type,
+                           RopeDivisors>::value,
+              "qkv_rope_lean_f32 must take the divisor table as its first parameter");
 static_assert(std::is_same<FirstParameter<decltype(&qkv_rope_wave<float, 128, kStorePlain, 4, false>)>::type,
                            RopeDivisors>::value,
               "qkv_rope_wave must take the divisor table as its first parameter");
@@ -865,6 +998,26 @@ static int rope_decode(void* qkv_, int batch, int head_num, int kv_head_num, int
     return note_launch(hipGetLastError());
 }
 
+// Workgroup shape for the one-vector-per-lane kernels, whose waves carry `wave_heads` whole heads each.
+// Head counts in whole groups of eight waves: 8 waves, all of one plane (q, k or v).  Otherwise `split`:
+// every wave places its own heads, and the workgroup has the largest number of waves from 8 down to 3 that
+// divides the token's waves, so that no wave is launched without heads (36 heads of fp16 in 512-thread
+// workgroups, 7 of 16 waves idle, measured 10 % slower than the general kernel).  waves = 0: the head
+// counts fit neither, the caller uses the general kernel.
+struct LeanShape {
+    int waves;
+    bool split;
+    int groups(int qkv_heads, int wave_heads) const { return (qkv_heads + wave_heads * waves - 1) / (wave_heads * waves); }
+};
+static LeanShape lean_shape(int head_num, int kv_head_num, int wave_heads) {
+    if (head_num % wave_heads != 0 || kv_head_num % wave_heads != 0) return {0, false};
+    if (head_num % (8 * wave_heads) == 0 && kv_head_num % (8 * wave_heads) == 0) return {8, false};
+    const int token_waves = (head_num + 2 * kv_head_num) / wave_heads;
+    for (int w = 8; w >= 3; w--)
+        if (token_waves % w == 0) return {w, true};
+    return {0, false};
+}
+
 // `append`: also (k_ / v_ non-NULL) or only (k_ / v_ NULL) write the k and v rows into the KV cache
 // [layers, batch, kv_head_num, max_seq_len, head_size] at layer `layer`.
 template <typename T>
@@ -952,17 +1105,21 @@ static int qkv_rope(void* q_, void* k_, void* v_, const void* qkv_, const void* 
     const bool positions_ok = (unsigned long long)batch * (unsigned long long)seq_len <= 0x7fffffffull;
     const unsigned positions = positions_ok ? (unsigned)batch * (unsigned)seq_len : 0u;
     const FastDiv fd = make_fastdiv((unsigned)seq_len);
-    // lean kernel: fp16, 128-element heads fully rotated, whole groups of 32 q / k / v heads, offsets
-    // inside a group and positions inside the batch in 32 bits; ISP_TUNE_QKV_WAVES = 1, 2, 4 opts out
+    // one-vector-per-lane kernels: 128-element heads fully rotated, head counts that fill whole waves (4 heads
+    // in fp16, 2 in fp32), offsets inside a group and positions inside the batch in 32 bits;
+    // ISP_TUNE_QKV_WAVES = 1, 2, 4 opts out
     const int waves_knob = tuning(ISP_TUNE_QKV_WAVES);
-    const bool lean_ok = sizeof(T) == 2 && vec_ok && head_size == 128 && rot == 128 &&
-                         head_num % 32 == 0 && kv_head_num % 32 == 0 &&
-                         (head_num + 2 * kv_head_num) / 32 <= 65535 &&
-                         (unsigned long long)seq_len * 256ull * 32ull <= 0xffffffffull &&
-                         (unsigned long long)max_seq_len * 256ull * 32ull <= 0xffffffffull &&
+    const int qkv_heads = head_num + 2 * kv_head_num;
+    const int lean_wave_heads = sizeof(T) == 2 ? 4 : 2;
+    const LeanShape lean = lean_shape(head_num, kv_head_num, lean_wave_heads);
+    const bool lean_ok = vec_ok && head_size == 128 && rot == 128 && lean.waves > 0 &&
+                         lean.groups(qkv_heads, lean_wave_heads) <= 65535 &&
+                         (unsigned long long)seq_len * 8192ull <= 0xffffffffull &&
+                         (unsigned long long)max_seq_len * 8192ull <= 0xffffffffull &&
                          positions_ok && (waves_knob <= 0 || waves_knob >= 8);
-    if (lean_ok) {
-        const dim3 g2((unsigned)token_num, (unsigned)((head_num + 2 * kv_head_num) / 32));
+    const dim3 lean_grid((unsigned)token_num, (unsigned)(lean_ok ? lean.groups(qkv_heads, lean_wave_heads) : 1));
+    const dim3 lean_block(64u * (unsigned)(lean_ok ? lean.waves : 1));
+    if (lean_ok && sizeof(T) == 2) {
         __half* qh = reinterpret_cast<__half*>(q);
         __half* kh = reinterpret_cast<__half*>(k);
         __half* vh = reinterpret_cast<__half*>(v);
@@ -971,10 +1128,15 @@ static int qkv_rope(void* q_, void* k_, void* v_, const void* qkv_, const void* 
         KvAppend<__half> aph = {reinterpret_cast<__half*>(ap.k_cache), reinterpret_cast<__half*>(ap.v_cache),
                                 ap.input_length, ap.max_seq_len};
         const bool with_append = aph.k_cache != nullptr;
+#define ISP_QKV_LEAN_3(K, B, A, S)                                                                 \
+    hipLaunchKernelGGL((qkv_rope_lean_f16<K, B, A, S>), lean_grid, lean_block, 0, s, tab, qh, kh,  \
+                       vh, xh, bh, padding_offset, history_length, positions, fd,                  \
+                       (unsigned)head_num, (unsigned)kv_head_num, aph)
 #define ISP_QKV_LEAN_2(K, B, A)                                                                    \
-    hipLaunchKernelGGL((qkv_rope_lean_f16<K, B, A>), g2, dim3(512), 0, s, tab, qh, kh, vh, xh, bh,  \
-                       padding_offset, history_length, positions, fd, (unsigned)head_num,          \
-                       (unsigned)kv_head_num, aph)
+    do {                                                                                           \
+        if (lean.split) ISP_QKV_LEAN_3(K, B, A, true);                                             \
+        else ISP_QKV_LEAN_3(K, B, A, false);                                                       \
+    } while (0)
 #define ISP_QKV_LEAN(K)                                                                            \
     do {                                                                                           \
         if (bh && with_append) ISP_QKV_LEAN_2(K, true, true);                                      \
@@ -985,8 +1147,42 @@ static int qkv_rope(void* q_, void* k_, void* v_, const void* qkv_, const void* 
         if (kind == kStoreThrough) ISP_QKV_LEAN(kStoreThrough);
         else if (kind == kStoreStream) ISP_QKV_LEAN(kStoreStream);
         else ISP_QKV_LEAN(kStorePlain);
+#undef ISP_QKV_LEAN_3
 #undef ISP_QKV_LEAN_2
 #undef ISP_QKV_LEAN
+        e = hipGetLastError();
+    } else if (lean_ok) {
+        // fp32 rows of 512 bytes: 16 heads per workgroup of 512 threads
+        float* qf = reinterpret_cast<float*>(q);
+        float* kf = reinterpret_cast<float*>(k);
+        float* vf = reinterpret_cast<float*>(v);
+        const float* xf = reinterpret_cast<const float*>(qkv);
+        const float* bf = reinterpret_cast<const float*>(bias);
+        KvAppend<float> apf = {reinterpret_cast<float*>(ap.k_cache), reinterpret_cast<float*>(ap.v_cache),
+                               ap.input_length, ap.max_seq_len};
+        const bool with_append = apf.k_cache != nullptr;
+#define ISP_QKV_LEAN32_3(K, B, A, S)                                                               \
+    hipLaunchKernelGGL((qkv_rope_lean_f32<K, B, A, S>), lean_grid, lean_block, 0, s, tab, qf, kf,  \
+                       vf, xf, bf, padding_offset, history_length, positions, fd,                  \
+                       (unsigned)head_num, (unsigned)kv_head_num, apf)
+#define ISP_QKV_LEAN32_2(K, B, A)                                                                  \
+    do {                                                                                           \
+        if (lean.split) ISP_QKV_LEAN32_3(K, B, A, true);                                           \
+        else ISP_QKV_LEAN32_3(K, B, A, false);                                                     \
+    } while (0)
+#define ISP_QKV_LEAN32(K)                                                                          \
+    do {                                                                                           \
+        if (bf && with_append) ISP_QKV_LEAN32_2(K, true, true);                                    \
+        else if (bf) ISP_QKV_LEAN32_2(K, true, false);                                             \
+        else if (with_append) ISP_QKV_LEAN32_2(K, false, true);                                    \
+        else ISP_QKV_LEAN32_2(K, false, false);                                                    \
+    } while (0)
+        if (kind == kStoreThrough) ISP_QKV_LEAN32(kStoreThrough);
+        else if (kind == kStoreStream) ISP_QKV_LEAN32(kStoreStream);
+        else ISP_QKV_LEAN32(kStorePlain);
+#undef ISP_QKV_LEAN32_3
+#undef ISP_QKV_LEAN32_2
+#undef ISP_QKV_LEAN32
         e = hipGetLastError();
     } else if (vec_ok && positions_ok && head_size == 128 && head_num + 2 * kv_head_num <= head_groups_max) {
         ISP_QKV_LAUNCH_WAVE(128);

@@ -200,12 +200,14 @@ def test_norm_rows_do_not_depend_on_the_batch_they_are_in(isp, dtype):
 
 
 @pytest.mark.parametrize("dtype", [np.float16, np.float32])
-@pytest.mark.parametrize("hs", [64, 128])
-def test_qkv_every_head_size_store_kind_and_wave_count(isp, dtype, hs):
+@pytest.mark.parametrize("hs,hn,kvn", [(64, 16, 8), (128, 12, 4), (128, 32, 32)])
+def test_qkv_every_head_size_store_kind_and_wave_count(isp, dtype, hs, hn, kvn):
     from inferspore_amd import capi
     # 64-element heads in whole groups of 8: the automatic choice in fp16 is the two-tokens-per-workgroup
-    # kernel, knob 8 the whole-row kernel, 1 / 2 / 4 the general one -- all must agree to the bit
-    batch, seq, hn, kvn = (3, 16, 16, 8) if hs == 64 else (3, 16, 12, 4)
+    # kernel, knob 8 the whole-row kernel, 1 / 2 / 4 the general one; 128-element heads in whole groups of 32
+    # (fp16) or 16 (fp32): automatic and knob 8 are the one-vector-per-lane kernels, 1 / 2 / 4 the general
+    # one -- all must agree to the bit
+    batch, seq = 3, 16
     lens, qkv, bias, po, hist = qkv_inputs(batch, seq, hn, kvn, hs, dtype, seed=hs, min_len=2)
     hist = np.array([0, 9, 300], np.int32)
     d_in, d_bias, d_hist, d_lens = dev(qkv), dev(bias), dev(hist), dev(lens)

@@ -55,7 +55,8 @@ def _run_pair(isp, dtype, batch, seq, hn, kvn, hs, rot, max_seq, layers, layer, 
 @pytest.mark.parametrize("batch,seq,hn,kvn,hs,rot,max_seq", [
     (8, 512, 32, 32, 128, 128, 1024),   # the benchmark configuration: the one-vector-per-lane kernel in fp16
     (3, 12, 64, 32, 128, 128, 40),      # same kernel, two q groups
-    (2, 9, 8, 2, 128, 128, 16),         # GQA: the general kernel
+    (2, 9, 8, 2, 128, 128, 16),         # GQA: every wave places its own heads
+    (2, 9, 6, 3, 128, 128, 16),         # head counts that fit no vector layout of whole waves: the general kernel
     (2, 9, 5, 1, 128, 64, 16),          # MQA, partial rotary
     (3, 7, 4, 2, 64, 64, 12),           # 64-element heads
     (3, 7, 16, 8, 64, 64, 12),          # 64-element heads in groups of 8: two tokens per workgroup in fp16

@@ -308,10 +308,16 @@ def test_qkv_rope_known_answer(isp):
 @pytest.mark.parametrize("dtype", [np.float16, np.float32])
 @pytest.mark.parametrize("batch,seq,hn,kvn,hs,rot", [
     (3, 12, 4, 4, 128, 128),    # vector path, tiny
-    (2, 9, 8, 2, 128, 128),     # GQA
-    (2, 9, 32, 8, 128, 128),    # GQA 32q/8kv: one whole q group, one group holding k, v and dead rows
+    (2, 9, 8, 2, 128, 128),     # GQA: q, k and v waves in one workgroup, the rest of it without heads
+    (2, 9, 32, 8, 128, 128),    # GQA 32q/8kv: one whole q group, one group holding k, v and waves without heads
     (2, 5, 40, 40, 128, 128),   # 120 heads: groups straddle the q/k and k/v boundaries
     (1, 7, 64, 8, 128, 128),    # 64q/8kv
+    (2, 9, 32, 16, 128, 128),   # fp32: whole groups of 16 heads (q, q, k, v groups); fp16: k and v share a workgroup
+    (2, 5, 48, 16, 128, 128),   # fp32: three q groups; fp16: q and k meet inside the second workgroup
+    (2, 5, 6, 2, 128, 128),     # multiples of 2: per-wave placement in fp32, the general kernel in fp16
+    (2, 5, 8, 4, 128, 128),     # fp16: 4 waves per token in one workgroup
+    (2, 5, 20, 4, 128, 128),    # fp16: 7 waves per token in one workgroup
+    (2, 5, 36, 4, 128, 128),    # fp16: 11 waves per token divide into no workgroup size: the general kernel
     (2, 6, 33, 3, 128, 128),    # head counts that are multiples of nothing
     (2, 9, 5, 1, 128, 64),      # MQA, partial rotary, head counts that do not fill a wave pass
     (3, 7, 4, 2, 64, 64),       # 64-wide heads
