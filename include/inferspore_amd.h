@@ -302,10 +302,10 @@ typedef enum isp_tuning_knob {
     ISP_TUNE_QKV_STORE = 6,          /* 1 = plain, 2 = non-temporal, 3 = write-through (default) */
     ISP_TUNE_QKV_WAVES = 7,          /* 1, 2 or 4: the general kernel with that many waves (groups of 8 heads) per
                                         workgroup; 8: as 0, but 64-element fp16 heads take the one-token whole-row
-                                        kernel; 0 = automatic: the fp16 one-vector-per-lane kernels where the shape
+                                        kernel; 0 = automatic: the one-vector-per-lane kernels where the shape
                                         allows them (128-element heads fully rotated with head counts multiples of
-                                        32; 64-element heads fully rotated with head counts multiples of 8), else
-                                        the general kernel with 4 waves */
+                                        4 in fp16, of 2 in fp32; 64-element fp16 heads fully rotated with head
+                                        counts multiples of 8), else the general kernel with 4 waves */
     ISP_TUNE_NORM_BLOCK_THREADS = 8, /* 256, 512 or 1024 threads per workgroup (several token rows share a
                                         workgroup when a row needs fewer); 0 = automatic */
     ISP_TUNE_NORM_ORDER = 9,         /* 2 = streaming (each vector processed, and the residual stored, as it
