@@ -329,7 +329,7 @@ def make_workloads(torch, lib, stream_handle, rotate):
         batch, seq, tokens, lens_d, po = padded_batch()
         hn, hs = 32, 128
         w.name, w.dtype, w.tokens = "transpose_remove_padding_f16_b8_s512", "f16", tokens
-        w.kernel = "isp::transpose_remove_padding_vec<512>"
+        w.kernel = "isp::transpose_remove_padding_vec<64>"
         w.bytes_per_launch = tokens * (2 * hn * hs * 2 + 4)
         R = w.sets_for(batch * hn * seq * hs * 2 + tokens * hn * hs * 2, rotate)
         srcs = [torch.randn((batch, hn, seq, hs), device=dev).to(torch.float16) for _ in range(R)]

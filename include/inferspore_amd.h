@@ -314,7 +314,8 @@ typedef enum isp_tuning_knob {
                                         4 / 5 = as 0, but a call with a residual and no bias never / always waits
                                         for a gamma vector where the bias vector would arrive (by default it does
                                         where the launch is one round of waves reading more than 24 MiB) */
-    ISP_TUNE_MOVER_BLOCK_THREADS = 10, /* KV append / broadcast: 256, 512 or 1024 threads per workgroup */
+    ISP_TUNE_MOVER_BLOCK_THREADS = 10, /* KV append / broadcast: 64, 128, 256 (default), 512 or 1024 threads per
+                                          workgroup; transpose-out: 64 (default), 128, 256 or 512 */
     ISP_TUNE_COUNT = 11
 } isp_tuning_knob;
 int isp_tuning_set(int knob, int value);

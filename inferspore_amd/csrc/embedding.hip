@@ -4,8 +4,8 @@
 // element type (the row is handled as bytes) and the result is bit-exact by construction.
 // Design: the token id is read once per workgroup into a scalar register (the reference re-reads
 // ids[] and does a div/mod for every 2-byte element) and the row moves as 16-byte vectors, one
-// vector per lane, one 4 KiB chunk of a row per workgroup -- the access order that streams best on
-// this memory system; wave-per-row and workgroup-per-row variants remain selectable for sweeps.
+// vector per lane, one 1 KiB chunk of a row per single-wave workgroup -- the access order that streams
+// best on this memory system; wave-per-row and workgroup-per-row variants remain selectable for sweeps.
 #include "isp_common.h"
 
 namespace isp {
@@ -48,15 +48,19 @@ __global__ __launch_bounds__(kBlock) void gather_rows_vec(const int32_t* __restr
     }
 }
 
-// One 16-byte vector per lane: a workgroup moves one 4 KiB chunk of one row.
+// One 16-byte vector per lane: a workgroup is a single wave and moves one 1 KiB chunk of one row.  A wave
+// that is its own workgroup starts as soon as any wave slot is free; measured against 256-thread
+// workgroups (4 KiB chunks) on 8192 rows of fp16: 4096 wide 22.4 against 23.2 us, 5120 wide (whose third
+// 4 KiB chunk is half empty) 28.4 against 29.0, 3072 wide 18.0 against 20.2; 128, 192, 320 ... 512 threads
+// all lie between or behind.
 template <int ST>
-__global__ __launch_bounds__(kBlock) void gather_chunks_vec(const int32_t* __restrict__ ids,
-                                                            char* __restrict__ out,
-                                                            const char* __restrict__ table,
-                                                            unsigned chunks_per_row,
-                                                            unsigned row_vec, int vocab) {
+__global__ __launch_bounds__(kWave) void gather_chunks_vec(const int32_t* __restrict__ ids,
+                                                           char* __restrict__ out,
+                                                           const char* __restrict__ table,
+                                                           unsigned chunks_per_row,
+                                                           unsigned row_vec, int vocab) {
     const unsigned row = blockIdx.x / chunks_per_row;
-    const unsigned v = (blockIdx.x % chunks_per_row) * kBlock + threadIdx.x;
+    const unsigned v = (blockIdx.x % chunks_per_row) * kWave + threadIdx.x;
     if (v >= row_vec) return;
     const int id = __builtin_amdgcn_readfirstlane(ids[row]);
     const bool in_range = vocab <= 0 || (id >= 0 && id < vocab);
@@ -84,16 +88,16 @@ template <int ST>
 static void launch_gather(int variant, const int32_t* ids, char* o, const char* t, int tokens,
                           unsigned row_vec, int vocab, hipStream_t s) {
     const dim3 block(kBlock);
-    const size_t chunks = (row_vec + kBlock - 1) / kBlock;
+    const size_t chunks = (row_vec + kWave - 1) / kWave;
     if (variant == 1) {  // one wave per row
         hipLaunchKernelGGL((gather_rows_vec<kWave, 4, ST>), dim3((unsigned)((tokens + 3) / 4)), block, 0, s,
                            ids, o, t, tokens, row_vec, vocab);
     } else if (variant == 2 || (size_t)tokens * chunks > 0x7fffffffull) {  // one workgroup per row
         hipLaunchKernelGGL((gather_rows_vec<kBlock, 2, ST>), dim3((unsigned)tokens), block, 0, s, ids, o, t,
                            tokens, row_vec, vocab);
-    } else {  // one 4 KiB chunk of a row per workgroup, one vector per lane
-        hipLaunchKernelGGL((gather_chunks_vec<ST>), dim3((unsigned)((size_t)tokens * chunks)), block, 0, s,
-                           ids, o, t, (unsigned)chunks, row_vec, vocab);
+    } else {  // one 1 KiB chunk of a row per single-wave workgroup, one vector per lane
+        hipLaunchKernelGGL((gather_chunks_vec<ST>), dim3((unsigned)((size_t)tokens * chunks)), dim3(kWave), 0,
+                           s, ids, o, t, (unsigned)chunks, row_vec, vocab);
     }
 }
 

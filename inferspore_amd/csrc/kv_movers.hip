@@ -45,7 +45,7 @@ static SegSplit make_split(unsigned seg_vec) {
 }
 
 // dst[token, h, :] = src[b, h, s, :],  token + padding_offset[token] = b * seq_len + s.
-// grid = tokens * chunks, a chunk being 256 vectors of the token's heads*seg_vec vectors
+// grid = tokens * chunks, a chunk being BLOCK vectors of the token's heads*seg_vec vectors
 template <int BLOCK>
 __global__ __launch_bounds__(BLOCK) void transpose_remove_padding_vec(
     const char* __restrict__ src, const int32_t* __restrict__ padding_offset, char* __restrict__ dst,
@@ -187,10 +187,10 @@ __global__ __launch_bounds__(kBlock) void repeat_kv_units(
 
 constexpr long long kMaxGridYZ = 65535;
 
-// Threads per workgroup of the cache movers: 256, 512 or 1024 (tuning knob, else the measured default).
+// Threads per workgroup of the cache movers: 64 ... 1024 (tuning knob, else the measured default).
 static int mover_block() {
     const int knob = tuning(ISP_TUNE_MOVER_BLOCK_THREADS);
-    return (knob == 256 || knob == 512 || knob == 1024) ? knob : 256;
+    return (knob == 64 || knob == 128 || knob == 256 || knob == 512 || knob == 1024) ? knob : 256;
 }
 
 static int transpose_remove_padding(const void* src, const int32_t* padding_offset, void* dst,
@@ -204,11 +204,11 @@ static int transpose_remove_padding(const void* src, const int32_t* padding_offs
     ISP_REQUIRE_PTR(dst);
     const size_t seg = (size_t)head_size * elem;
     const size_t row_vec = (size_t)head_num * (seg / 16);
-    // one 512-thread workgroup per token when a token's row is exactly that (32 heads of 256 bytes): 9.54
-    // against 9.79 us; with two such workgroups per token (64 heads) 256 threads stay 0.7 % ahead.  The knob
-    // of the cache movers overrides.
+    // single-wave workgroups: 9.17 us against 9.5-9.6 with 128, 256 or 512 threads at 2977 tokens of 32 heads
+    // (the two cache movers, whose grids hold workgroups that leave at once, measured 2-3 % slower that way
+    // and keep 256).  The knob of the cache movers overrides.
     const int knob = tuning(ISP_TUNE_MOVER_BLOCK_THREADS);
-    const int blk = (knob == 256 || knob == 512) ? knob : (row_vec == 512 ? 512 : 256);
+    const int blk = (knob == 64 || knob == 128 || knob == 256 || knob == 512) ? knob : 64;
     const size_t chunks = (row_vec + blk - 1) / blk;
     // the vector kernel keeps padded positions in 32 bits and divides with a multiply-high
     if (seg % 16 == 0 && aligned16(src) && aligned16(dst) && chunks * (size_t)token_num <= 0x7fffffffull &&
@@ -221,6 +221,8 @@ static int transpose_remove_padding(const void* src, const int32_t* padding_offs
                        (unsigned)batch * (unsigned)seq_len, head_num, make_fastdiv((unsigned)seq_len), \
                        make_split(seg_vec), make_fastdiv((unsigned)chunks))
         if (blk == 512) ISP_LAUNCH_TRANSPOSE(512);
+        else if (blk == 128) ISP_LAUNCH_TRANSPOSE(128);
+        else if (blk == 64) ISP_LAUNCH_TRANSPOSE(64);
         else ISP_LAUNCH_TRANSPOSE(256);
 #undef ISP_LAUNCH_TRANSPOSE
     } else {
@@ -273,6 +275,8 @@ static int concat_kv(const void* k_src, const void* v_src, void* k_cache, void* 
                        make_split(seg_vec), mg)
         if (blk == 1024) ISP_LAUNCH_CONCAT(1024);
         else if (blk == 512) ISP_LAUNCH_CONCAT(512);
+        else if (blk == 128) ISP_LAUNCH_CONCAT(128);
+        else if (blk == 64) ISP_LAUNCH_CONCAT(64);
         else ISP_LAUNCH_CONCAT(256);
 #undef ISP_LAUNCH_CONCAT
     } else {
@@ -326,6 +330,8 @@ static int repeat_kv(const void* k_cache, const void* v_cache, void* k_dst, void
                        kv_head_num, max_seq_len, max_k_len, make_split(seg_vec), mg)
         if (blk == 1024) ISP_LAUNCH_REPEAT(1024);
         else if (blk == 512) ISP_LAUNCH_REPEAT(512);
+        else if (blk == 128) ISP_LAUNCH_REPEAT(128);
+        else if (blk == 64) ISP_LAUNCH_REPEAT(64);
         else ISP_LAUNCH_REPEAT(256);
 #undef ISP_LAUNCH_REPEAT
     } else {

@@ -318,15 +318,15 @@ def test_kv_movers_every_workgroup_size(isp):
             ekd[b, h, :h0 + n] = ek[0, b, h // (hn // kvn), :h0 + n]
             evd[b, h, :h0 + n] = ev[0, b, h // (hn // kvn), :h0 + n]
     assert all(np.array_equal(a, b) for a, b in zip(base, (ek, ev, ekd, evd)))
-    for block in (256, 512, 1024):
+    for block in (64, 128, 256, 512, 1024):
         say("kv movers with %d-thread workgroups" % block)
         got = with_knobs({capi.TUNE_MOVER_BLOCK_THREADS: block}, run)
         assert all(np.array_equal(a, b) for a, b in zip(got, base))
 
 
 def test_transpose_out_every_workgroup_size(isp):
-    """32 heads of 256 bytes take one 512-thread workgroup per token by default, everything else 256-thread
-    ones; both sizes must move the same bytes for either shape."""
+    """Single-wave workgroups by default; every compiled workgroup size must move the same bytes, for a row that
+    is a whole number of the largest workgroups and for one that is not."""
     from inferspore_amd import capi
     for heads in (32, 40):
         batch, seq, hs = 3, 10, 128
@@ -345,7 +345,7 @@ def test_transpose_out_every_workgroup_size(isp):
         base = run()
         expect = np.concatenate([src[b, :, :n].permute(1, 0, 2).cpu().numpy() for b, n in enumerate(lens)])
         assert np.array_equal(base, expect)
-        for block in (256, 512):
+        for block in (64, 128, 256, 512):
             say("transpose-out, %d heads, %d-thread workgroups" % (heads, block))
             assert np.array_equal(with_knobs({capi.TUNE_MOVER_BLOCK_THREADS: block}, run), base)
 
