@@ -293,12 +293,11 @@ typedef enum isp_tuning_knob {
     ISP_TUNE_NORM_STORE = 1,         /* output stores: 1 = plain (default where a launch writes at most 1 MiB),
                                         2 = non-temporal (default otherwise), 3 = non-temporal write-through */
     ISP_TUNE_SWIGLU_UNROLL = 2,      /* 1 (default), 2 or 4 vector pairs in flight per lane */
-    ISP_TUNE_SWIGLU_STORE = 3,       /* 1 = plain, 2 = non-temporal (default), 3 = write-through (default for
-                                        outputs of 16-80 MiB) */
+    ISP_TUNE_SWIGLU_STORE = 3,       /* 1 = plain, 2 = non-temporal (default), 3 = write-through */
     ISP_TUNE_EMBED_VARIANT = 4,      /* 1 = a wave per row, 2 = a workgroup per row,
-                                        3 = a workgroup per 4 KiB chunk of a row (default) */
-    ISP_TUNE_EMBED_STORE = 5,        /* 1 = plain, 2 = non-temporal (default up to 8 MiB of output),
-                                        3 = write-through (default above) */
+                                        3 = a single-wave workgroup per 1 KiB chunk of a row (default) */
+    ISP_TUNE_EMBED_STORE = 5,        /* 1 = plain (default up to 1 MiB of output), 2 = non-temporal (default up to
+                                        8 MiB), 3 = write-through (default above) */
     ISP_TUNE_QKV_STORE = 6,          /* 1 = plain, 2 = non-temporal, 3 = write-through (default) */
     ISP_TUNE_QKV_WAVES = 7,          /* 1, 2 or 4: the general kernel with that many waves (groups of 8 heads) per
                                         workgroup; 8: as 0, but 64-element fp16 heads take the one-token whole-row

@@ -88,11 +88,9 @@ static int swiglu(const void* in_, void* out_, int tokens, int inter, hipStream_
     if (inter % VEC == 0 && aligned16(in) && aligned16(out) && total_vec < 0xffff0000ull) {
         int unroll = tuning(ISP_TUNE_SWIGLU_UNROLL);
         if (unroll != 1 && unroll != 2 && unroll != 4) unroll = 1;
-        // non-temporal stores, except for outputs of 16-80 MiB, where the write-through form measured 1-2 % faster
-        // (1024-2977 rows of 11008 fp16; 0.3-1 % slower from 4096 rows up, equal below)
-        const size_t written = total * sizeof(T);
-        const bool mid = written > ((size_t)16 << 20) && written < ((size_t)80 << 20);
-        const int kind = store_kind(tuning(ISP_TUNE_SWIGLU_STORE), mid ? kStoreThrough : kStoreStream);
+        // non-temporal stores: equal to or 1-2 % ahead of the write-through form at every size from 256 to 8192
+        // rows of 11008 in both precisions, 5-10 % ahead of ordinary stores from 1024 rows up
+        const int kind = store_kind(tuning(ISP_TUNE_SWIGLU_STORE), kStoreStream);
         const size_t per_block = (size_t)kWave * unroll;
         const dim3 grid((unsigned)((total_vec + per_block - 1) / per_block)), block(kWave);
         const unsigned nv = (unsigned)total_vec, vpr = (unsigned)(inter / VEC);
