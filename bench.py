@@ -568,7 +568,7 @@ def time_workload(torch, w, steps, warmup, regions, stream, gate):
     return {"wall_ms": wall_ms, "event_ms": per[len(per) // 2], "fastest": per[0], "slowest": per[-1],
             "queued_before_start": (host_at[regions] - t0) * 1e3 < gate_ms, "regions_ahead": ahead,
             "gate_launches": g, "issued": issued, "host_enqueue_us_per_launch": enqueue_us,
-            "host_us_per_launch_empty_queue": host_us}
+            "host_us_per_launch_empty_queue": host_us, "per_region_ms": per_all}
 
 
 def measure(torch, w, steps, warmup, regions, stream, traffic, gate):
