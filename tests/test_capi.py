@@ -147,3 +147,21 @@ def test_argument_validation_of_the_neighbour_entry_points(lib):
     assert lib.isp_calibration_copy(None, None, 0, None) == capi.OK
     assert lib.isp_tuning_set(99, 1) == capi.ERR_BAD_SHAPE
     assert lib.isp_tuning_set(capi.TUNE_NORM_STORE, 0) >= 0
+
+
+def test_build_flags_for_the_kernel_files():
+    """Every HIP compile switches packed-fp32 formation off; every kernel file of the C-ABI library is built with
+    preloaded kernel arguments except the general norm kernel, and the few-rows norm kernels -- the ones that
+    need the preloading most -- live in a file that gets it."""
+    from inferspore_amd import build
+    flags = build.HIPCC_FLAGS
+    i = flags.index("-packed-fp32-ops")
+    assert flags[i - 3:i] == ["-Xclang", "-target-feature", "-Xclang"]
+    assert "--offload-arch=gfx950" in flags
+    assert build.KERNARG_PRELOAD == ["-mllvm", "-amdgpu-kernarg-preload-count=16"]
+    kernel_files = sorted(f for f in os.listdir(build.CSRC) if f.endswith(".hip"))
+    assert "norm_few_rows.hip" in kernel_files and "norm.hip" in kernel_files
+    assert build.NO_KERNARG_PRELOAD == {"norm.hip"}
+    few = open(os.path.join(build.CSRC, "norm_few_rows.hip")).read()
+    assert "__global__" in few and "void fused_norm_few_rows(" in few
+    assert "void fused_norm_few_rows(" not in open(os.path.join(build.CSRC, "norm.hip")).read()
