@@ -122,15 +122,17 @@ class Workload:
         self.launch = launch
 
 
-def norm_kernel_name(lib, es, tokens, hidden, fused):
-    """The instantiation the launcher picks (`fused`: with residual and bias, as the benchmark's fused rows are)."""
+def norm_kernel_name(lib, es, tokens, hidden, fused, with_bias=None):
+    """The instantiation the launcher picks (`fused`: with a residual; `with_bias` defaults to `fused`)."""
+    with_bias = fused if with_bias is None else (fused and with_bias)
     v = [ctypes.c_int() for _ in range(4)]
     rc = lib.isp_norm_launch_config(es, tokens, hidden, int(fused), *[ctypes.byref(x) for x in v])
     if rc:
         return "isp::fused_norm_generic"
     t = "__half" if es == 2 else "float"
-    if lib.isp_norm_launch_variant(es, tokens, hidden, int(fused), int(fused), 0) == 1:
-        return "isp::fused_norm_few_rows<%s, %d, %d, %d, %d>" % (t, v[1].value, v[0].value, v[3].value, 2 if fused else 0)
+    if lib.isp_norm_launch_variant(es, tokens, hidden, int(fused), int(with_bias), 0) == 1:
+        return "isp::fused_norm_few_rows<%s, %d, %d, %d, %d>" % (t, v[1].value, v[0].value, v[3].value,
+                                                                 (2 if with_bias else 1) if fused else 0)
     return "isp::fused_norm_rows<%s, %d, %d, %d, %d>" % (t, v[1].value, v[0].value, v[3].value, v[2].value)
 
 
@@ -173,7 +175,7 @@ def make_workloads(torch, lib, stream_handle, rotate):
         bias = (0.02 * torch.randn(hidden, device=dev)).to(tdtype) if fused and with_bias else None
         gamma = (0.5 + torch.rand(hidden, device=dev)).to(tdtype)
         w.keep = (outs, ress, bias, gamma)
-        w.kernel = norm_kernel_name(lib, es, tokens, hidden, fused)
+        w.kernel = norm_kernel_name(lib, es, tokens, hidden, fused, with_bias)
         if fused:
             fn = getattr(lib, "isp_fused_add_bias_residual_rmsnorm_" + sfx)
             w.bind(fn, [(ress[j].data_ptr(), outs[j].data_ptr(), bias.data_ptr() if with_bias else None, gamma.data_ptr(),

@@ -282,7 +282,8 @@ int isp_norm_launch_config(int elem_size, int tokens, int hidden, int fused, int
 
 /* isp_norm_launch_variant: 1 if a call with these operands (`flags` as for the fused entry point) is launched
  *   as isp::fused_norm_few_rows -- the same row algorithm with the operand set fixed at compile time, taken by
- *   launches that occupy less than a quarter of the device (every decode-step norm) -- and 0 if as the general
+ *   launches whose waves are all resident at once (every decode-step norm, prefill batches of a few hundred
+ *   rows) unless they want the general kernel's pacing load -- and 0 if as the general
  *   isp::fused_norm_rows; the waves per row, vectors per lane and store kind are those of
  *   isp_norm_launch_config, the workgroup is max(256, 64 x waves per row) threads.  No counterpart in the
  *   reference (its launcher has one configuration, src/kernels/fused_addresidual_norm.cu:155-159). */

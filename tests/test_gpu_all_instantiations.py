@@ -136,7 +136,14 @@ def test_norm_pacing_load_gives_the_same_bits(isp, oracle, dtype):
     vec = 8 if dtype == np.float16 else 4
     for wpr, nv in ((1, 1), (2, 2), (4, 4), (8, 8), (16, 2)):
         hidden = vec * 64 * wpr * nv - (vec if nv > 1 else 0)
-        tokens = 300   # beyond the few-rows kernels for every split
+        # enough rows that the unpaced launch, too, takes the general kernel (the kernels with the operand set
+        # fixed at compile time take every launch whose waves are all resident at once, and have no pacing load)
+        tokens = 300
+        es = 2 if dtype == np.float16 else 4
+        unpaced = {capi.TUNE_NORM_WAVES_PER_ROW: wpr, capi.TUNE_NORM_ORDER: 4}
+        while with_knobs(unpaced, lambda: capi.lib().isp_norm_launch_variant(es, tokens, hidden, 1, 0, 0)) != 0:
+            tokens *= 2
+        assert tokens <= 20000
         res, out, _, gamma = norm_inputs(tokens, hidden, dtype, seed=7 * wpr + nv)
         d_gamma = dev(gamma)
 
