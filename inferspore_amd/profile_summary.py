@@ -193,6 +193,7 @@ def main():
     out = ["rocprofv3 kernel-trace summary: " + a.title, "",
            "command (run from /tmp with TMPDIR=/tmp on the MI355X box):",
            "  rocprofv3 --kernel-trace --stats --output-format csv -d RUN/trace -o bench -- python3 bench.py " + a.bench_args,
+           "  python3 bench.py " + a.bench_args + " > RUN/plain.json   (optional: the unprofiled table at the end)",
            "  python3 -m inferspore_amd.profile_summary RUN --out profiles" + extra,
            "  (--steps %d --warmup %d; launches rotate over >1 GiB of buffer sets; warm-up, gate and lead-in dispatches excluded)"
            % (steps, bench["warmup"]), "",
