@@ -409,6 +409,12 @@ def make_workloads(torch, lib, stream_handle, rotate):
         ("fused_add_residual_rmsnorm_f16_2977x4096_no_bias",
          lambda: norm("fused_add_residual_rmsnorm_f16_2977x4096_no_bias", 2977, 4096, torch.float16, True, False)),
         ("rmsnorm_f32_64x4096", lambda: norm("rmsnorm_f32_64x4096", 64, 4096, torch.float32, False)),
+        # a decode step's two norms at batch 16 and 256: launch-bound, the kernels with the operand set fixed at compile time
+        ("rmsnorm_f16_16x4096", lambda: norm("rmsnorm_f16_16x4096", 16, 4096, torch.float16, False)),
+        ("fused_add_residual_rmsnorm_f16_16x4096_no_bias",
+         lambda: norm("fused_add_residual_rmsnorm_f16_16x4096_no_bias", 16, 4096, torch.float16, True, False)),
+        ("fused_add_residual_rmsnorm_f16_256x4096_no_bias",
+         lambda: norm("fused_add_residual_rmsnorm_f16_256x4096_no_bias", 256, 4096, torch.float16, True, False)),
         ("rmsnorm_f32_16384x4096", lambda: norm("rmsnorm_f32_16384x4096", 16384, 4096, torch.float32, False)),
         ("embedding_f16_8192x4096_v32000", embedding),
         ("qkv_bias_rope_transpose_f16_b8_s512", qkv),
