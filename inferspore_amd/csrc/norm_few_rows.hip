@@ -1,4 +1,5 @@
-// RMSNorm and fused add-residual + RMSNorm for launches of a few rows (every decode-step norm) on gfx950.
+// RMSNorm and fused add-residual + RMSNorm for launches of a few rows -- every decode-step norm, and prefill
+// batches up to the size whose waves are all resident at once -- on gfx950.
 // Semantics and row algorithm: norm_rows.h (src/kernels/fused_addresidual_norm.cu:55-97 in the reference).
 // This file is built with kernel-argument preloading like the other kernel files: the arguments arrive in scalar
 // registers with the wave instead of being fetched by its first instructions, one round trip less in a launch

@@ -1,5 +1,5 @@
 // Device code shared by the RMSNorm kernels (norm.hip: the general kernel and the launchers; norm_few_rows.hip:
-// the kernels that launches of a few rows take).  The two live in separate translation units because they are
+// the kernels that launches of a few rows -- all of whose waves are resident at once -- take).  The two live in separate translation units because they are
 // compiled differently: the few-rows kernels with their arguments preloaded into scalar registers at wave
 // start, the general kernel without.
 #pragma once
