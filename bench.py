@@ -267,15 +267,18 @@ def make_workloads(torch, lib, stream_handle, rotate):
                     "head_dim": hs}
         return w
 
-    def qkv_append(fused):
+    def qkv_append(fused, with_bias=True):
         """QKV step + KV-cache append at the benchmark shape: one fused launch (k and v rows written to the
         cache only), or the two launches it replaces.  Both are priced at the bytes the fused form has
-        to move (packed qkv read once; q and the cache rows written once)."""
+        to move (packed qkv read once; q and the cache rows written once).  `with_bias=False` (fused form only)
+        is the call a LLaMA layer makes."""
         w = Workload()
         tdtype, es, hn, kvn, hs, max_seq = torch.float16, 2, 32, 32, 128, 1024
         batch, seq, tokens, lens_d, po = padded_batch()
         w.dtype, w.tokens = "f16", tokens
-        w.bytes_per_launch = tokens * (2 * (hn + 2 * kvn) * hs * es + 4) + (hn + 2 * kvn) * hs * es + 3 * batch * 4
+        w.bytes_per_launch = tokens * (2 * (hn + 2 * kvn) * hs * es + 4) + 3 * batch * 4
+        if with_bias:
+            w.bytes_per_launch += (hn + 2 * kvn) * hs * es
         hist = torch.zeros(batch, device=dev, dtype=torch.int32)
         bias = (0.02 * torch.randn((hn + 2 * kvn) * hs, device=dev)).to(tdtype)
         set_bytes = tokens * (hn + 2 * kvn) * hs * es + batch * hn * seq * hs * es + 2 * batch * kvn * max_seq * hs * es
@@ -287,10 +290,11 @@ def make_workloads(torch, lib, stream_handle, rotate):
         caches = [[torch.zeros((1, batch, kvn, max_seq, hs), device=dev, dtype=tdtype) for _ in range(2)] for _ in range(R)]
         w.keep = (lens_d, po, hist, bias, ins, qs, caches)
         if fused:
-            w.name, w.kernel = "qkv_bias_rope_transpose_append_f16_b8_s512_S1024", "isp::qkv_rope_lean_f16<2, true, true, false>"
+            w.name = "qkv_bias_rope_transpose_append_f16_b8_s512_S1024" + ("" if with_bias else "_no_bias")
+            w.kernel = "isp::qkv_rope_lean_f16<2, %s, true, false>" % ("true" if with_bias else "false")
             w.bind(lib.isp_qkv_bias_rope_transpose_append_f16,
                    [(qs[j].data_ptr(), None, None, caches[j][0].data_ptr(), caches[j][1].data_ptr(), 0, max_seq,
-                     ins[j].data_ptr(), bias.data_ptr(), po.data_ptr(), hist.data_ptr(), lens_d.data_ptr(), batch, seq,
+                     ins[j].data_ptr(), bias.data_ptr() if with_bias else None, po.data_ptr(), hist.data_ptr(), lens_d.data_ptr(), batch, seq,
                      tokens, hn, kvn, hs, hs, 10000.0, st) for j in range(R)])
         else:
             w.name = "qkv_bias_rope_transpose_then_concat_kv_f16_b8_s512_S1024"
@@ -421,6 +425,7 @@ def make_workloads(torch, lib, stream_handle, rotate):
         # the same step as LLaMA runs it: its projections have no bias (layer_weights.cc:58-62 sets the pointers to null)
         ("qkv_bias_rope_transpose_f16_b8_s512_no_bias", lambda: qkv(tag="_no_bias", with_bias=False)),
         ("qkv_bias_rope_transpose_append_f16_b8_s512_S1024", lambda: qkv_append(True)),
+        ("qkv_bias_rope_transpose_append_f16_b8_s512_S1024_no_bias", lambda: qkv_append(True, with_bias=False)),
         ("qkv_bias_rope_transpose_then_concat_kv_f16_b8_s512_S1024", lambda: qkv_append(False)),
         ("swiglu_f16_prefill_8192x11008", lambda: swiglu(8192, "prefill")),
         ("swiglu_f16_decode_256x11008", lambda: swiglu(256, "decode")),
