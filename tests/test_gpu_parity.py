@@ -336,6 +336,26 @@ def test_qkv_rope_shapes(isp, oracle, dtype, batch, seq, hn, kvn, hs, rot):
     _check_qkv(isp, oracle, dtype, batch, seq, hn, kvn, hs, rot, with_bias=False, seed=3, min_len=1)
 
 
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+def test_qkv_rope_random_head_counts(isp, oracle, dtype):
+    """Thirty seeded draws of (query heads, key/value heads, batch, padded length, histories, bias or none) with
+    128-element heads: between them they take the one-vector-per-lane kernels with every workgroup size from
+    three to eight waves, per workgroup and per wave placement, and the general kernel for the head counts that
+    fit neither -- all against the oracle."""
+    rng = np.random.default_rng(2024 if dtype == np.float16 else 4202)
+    for case in range(30):
+        kvn = int(rng.choice([1, 2, 3, 4, 6, 8, 12, 16, 32]))
+        hn = kvn * int(rng.choice([1, 2, 3, 4, 8]))
+        if hn > 64:
+            hn = 64 // kvn * kvn
+        batch, seq = int(rng.integers(1, 5)), int(rng.integers(1, 20))
+        hist = rng.integers(0, 3000, size=batch).astype(np.int32)
+        with_bias = bool(rng.integers(0, 2))
+        say("qkv random %s case %d: hn=%d kvn=%d b=%d s=%d bias=%s" % (dtype.__name__, case, hn, kvn, batch, seq, with_bias))
+        _check_qkv(isp, oracle, dtype, batch, seq, hn, kvn, 128, 128, with_bias=with_bias, seed=1000 + case,
+                   min_len=0, history=hist)
+
+
 def test_qkv_rope_large_positions_fp32(isp, oracle):
     # history pushes timesteps to ~4000: the angle must still match the oracle's fp32 angle exactly
     _check_qkv(isp, oracle, np.float32, 2, 64, 4, 4, 128, 128, seed=8, history=[4000, 2500])
